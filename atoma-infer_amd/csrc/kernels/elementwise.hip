@@ -551,21 +551,27 @@ __device__ __forceinline__ int up_index(int i, int inter, int block) {
   return block ? ((i >> 4) << 5) + 16 + (i & 15) : inter + i;
 }
 
+// the gate's activation: 0 silu, 1 the tanh form of gelu, 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3)))
+__device__ __forceinline__ float gate_act(float g, int act) {
+  if (act == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  return g / (1.0f + expf(-g));
+}
+
 template <typename T>
-__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total, int block) {
+__global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, size_t total, int block, int act) {
   for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
     const size_t t = idx / inter;
     const int i = (int)(idx % inter);
     const float g = to_f32(gu[t * 2 * inter + gate_index(i, block)]);
     const float u = to_f32(gu[t * 2 * inter + up_index(i, inter, block)]);
-    out[idx] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    out[idx] = from_f32<T>(gate_act(g, act) * u);
   }
 }
 
 // four values per thread; needs inter % 4 == 0 and 16-byte aligned rows
 template <typename T>
 __global__ void __launch_bounds__(256)
-swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int n_tokens, int block) {
+swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int n_tokens, int block, int act) {
   const int quads = inter >> 2;
   const size_t total = (size_t)n_tokens * quads;
   for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
@@ -575,14 +581,14 @@ swiglu_vec_kernel(const T* __restrict__ gu, T* __restrict__ out, int inter, int 
     const f4 u = load4(gu + t * 2 * inter + up_index(i, inter, block));
     f4 o;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o.v[e] = g.v[e] / (1.0f + expf(-g.v[e])) * u.v[e];
+    for (int e = 0; e < 4; ++e) o.v[e] = gate_act(g.v[e], act) * u.v[e];
     store4(out + t * inter + i, o);
   }
 }
 
 // eight bfloat16 values per thread (16-byte loads and stores); needs inter % 8 == 0 and 16-byte aligned rows
 __global__ void __launch_bounds__(256)
-swiglu_vec8_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ out, int inter, int n_tokens, int block) {
+swiglu_vec8_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ out, int inter, int n_tokens, int block, int act) {
   const int octs = inter >> 3;
   const size_t total = (size_t)n_tokens * octs;
   for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
@@ -597,23 +603,23 @@ swiglu_vec8_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ out, 
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const float gv = bf16_bits_to_f32(g[e]);
-      o[e] = f32_to_bf16_bits(gv / (1.0f + expf(-gv)) * bf16_bits_to_f32(u[e]));
+      o[e] = f32_to_bf16_bits(gate_act(gv, act) * bf16_bits_to_f32(u[e]));
     }
     *reinterpret_cast<uint4*>(out + t * inter + i) = oraw;
   }
 }
 
-extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, int block,
+extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, int inter, int block, int act,
                             hipStream_t stream) {
   if (n_tokens <= 0) return 0;
-  if (block != 0 && (block != 16 || inter % 16)) return ATOMA_ERR_SHAPE;
+  if ((block != 0 && (block != 16 || inter % 16)) || act < 0 || act > 1) return ATOMA_ERR_SHAPE;
   const size_t total = (size_t)n_tokens * inter;
   if (dtype == kBF16 && inter % 8 == 0 && ((uintptr_t)gu & 15) == 0 && ((uintptr_t)out & 15) == 0) {
     size_t octs = total / 8;
     int vb = (int)((octs + 255) / 256);
     if (vb > 16384) vb = 16384;
     hipLaunchKernelGGL(swiglu_vec8_kernel, dim3(vb), dim3(256), 0, stream, (const uint16_t*)gu, (uint16_t*)out, inter,
-                       n_tokens, block);
+                       n_tokens, block, act);
     ATOMA_LAUNCH_CHECK();
     return 0;
   }
@@ -623,10 +629,10 @@ extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, 
     if (vb > 16384) vb = 16384;
     if (dtype == kF32)
       hipLaunchKernelGGL(swiglu_vec_kernel<float>, dim3(vb), dim3(256), 0, stream, (const float*)gu, (float*)out, inter,
-                         n_tokens, block);
+                         n_tokens, block, act);
     else if (dtype == kBF16)
       hipLaunchKernelGGL(swiglu_vec_kernel<bf16_t>, dim3(vb), dim3(256), 0, stream, (const bf16_t*)gu, (bf16_t*)out,
-                         inter, n_tokens, block);
+                         inter, n_tokens, block, act);
     else
       return ATOMA_ERR_DTYPE;
     ATOMA_LAUNCH_CHECK();
@@ -636,10 +642,10 @@ extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, 
   if (blocks > 65536) blocks = 65536;
   if (dtype == kF32)
     hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)gu, (float*)out, inter,
-                       total, block);
+                       total, block, act);
   else if (dtype == kBF16)
     hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3(blocks), dim3(256), 0, stream, (const bf16_t*)gu, (bf16_t*)out,
-                       inter, total, block);
+                       inter, total, block, act);
   else
     return ATOMA_ERR_DTYPE;
   ATOMA_LAUNCH_CHECK();

@@ -1,7 +1,9 @@
 // Feed-forward layers that route every token to a few of many experts.
 //
-//   route_topk    per token: scores = sigmoid(router logits) in float32, the `top` largest (the lower index wins a
-//                 tie) with their scores: a (token, choice) pair is a "slot", numbered token * top + choice;
+//   route_topk    per token: scores = sigmoid(router logits), or their softmax over all experts, in float32; the `top`
+//                 experts with the largest score + correction[expert] (no correction: the score alone; the lower
+//                 index wins a tie) with their weights, score * scale (the correction chooses, it does not weigh):
+//                 a (token, choice) pair is a "slot", numbered token * top + choice;
 //   route_group   one workgroup: slots ordered by expert (perm), where each expert's slots start (offsets), and the
 //                 list of row tiles (expert, first place in perm) that the products below walk.  Which place a slot
 //                 gets inside its expert's range is not fixed; no result depends on it, since every row of a product
@@ -11,6 +13,8 @@
 //                 depend on the batch around it.  src is the slot's token (first product: the token's input, times its
 //                 score) or the slot itself (second product); the second product writes choice c of token t to row
 //                 c * T + t, so that the choices of a token lie in planes which the next norm adds in order.
+//                 act = 2 squares what is positive of a result and drops the rest (experts without a gate: relu^2);
+//                 out_scale[slot] multiplies a result (experts whose weight applies to their output).
 #include "common.h"
 
 using namespace atoma;
@@ -19,38 +23,66 @@ constexpr int kTileM = 64, kTileN = 64, kStepK = 16;
 
 __global__ void __launch_bounds__(256)
 route_topk_kernel(const float* __restrict__ logits, int ld, int experts, int top, int32_t* __restrict__ ids,
-                  float* __restrict__ weights, int n_tokens) {
+                  float* __restrict__ weights, int n_tokens, int softmax, const float* __restrict__ correction,
+                  float scale) {
   // a wave a token; lane l holds experts l, l + 64, ...
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= n_tokens) return;
   constexpr int PER = 16;      // experts <= 1024
-  float sc[PER];
+  // sc: what chooses (score, plus the correction where there is one); wt: what weighs (the score alone)
+  float sc[PER], wt[PER];
+  if (softmax) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = lane + j * 64;
+      wt[j] = e < experts ? logits[(size_t)t * ld + e] : -INFINITY;
+      mx = fmaxf(mx, wt[j]);
+    }
+    mx = wave_max(mx);
+    float sum = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      wt[j] = lane + j * 64 < experts ? expf(wt[j] - mx) : 0.f;
+      sum += wt[j];
+    }
+    sum = wave_sum(sum);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) wt[j] /= sum;
+  } else {
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = lane + j * 64;
+      wt[j] = e < experts ? 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e])) : 0.f;
+    }
+  }
 #pragma unroll
   for (int j = 0; j < PER; ++j) {
     const int e = lane + j * 64;
-    sc[j] = e < experts ? 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e])) : -1.f;
+    sc[j] = e < experts ? (correction != nullptr ? wt[j] + correction[e] : wt[j]) : -INFINITY;
   }
   for (int c = 0; c < top; ++c) {
-    float best = -2.f;
+    float best = -INFINITY, bw = 0.f;
     int arg = 0x7fffffff;
 #pragma unroll
     for (int j = 0; j < PER; ++j)
-      if (sc[j] > best) best = sc[j], arg = lane + j * 64;
+      if (sc[j] > best) best = sc[j], bw = wt[j], arg = lane + j * 64;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
       const float ob = __shfl_xor(best, off, 64);
+      const float ow = __shfl_xor(bw, off, 64);
       const int oa = __shfl_xor(arg, off, 64);
-      if (ob > best || (ob == best && oa < arg)) best = ob, arg = oa;
+      if (ob > best || (ob == best && oa < arg)) best = ob, bw = ow, arg = oa;
     }
-    if (arg >= experts) arg = c;     // logits that are no numbers: still an expert of the layer
+    if (arg >= experts) arg = c, bw = 0.f;     // logits that are no numbers: still an expert of the layer
     if (lane == 0) {
       ids[(size_t)t * top + c] = arg;
-      weights[(size_t)t * top + c] = best;
+      weights[(size_t)t * top + c] = bw * scale;
     }
 #pragma unroll
     for (int j = 0; j < PER; ++j)
-      if (lane + j * 64 == arg) sc[j] = -1.f;
+      if (lane + j * 64 == arg) sc[j] = -INFINITY;
   }
 }
 
@@ -87,7 +119,8 @@ __global__ void __launch_bounds__(256)
 expert_gemm_kernel(const TA* __restrict__ a, int lda, int a_div, const float* __restrict__ scale,
                    const TW* __restrict__ w, TC* __restrict__ c, int ldc, int N, int K,
                    const int32_t* __restrict__ perm, const int32_t* __restrict__ offsets,
-                   const int32_t* __restrict__ tiles, int top, int plane_rows) {
+                   const int32_t* __restrict__ tiles, int top, int plane_rows, int act,
+                   const float* __restrict__ out_scale) {
   __shared__ float as[kStepK][kTileM + 4];
   __shared__ float ws[kStepK][kTileN + 4];
   __shared__ int32_t slot_of[kTileM];
@@ -134,10 +167,13 @@ expert_gemm_kernel(const TA* __restrict__ a, int lda, int a_div, const float* __
     const int slot = slot_of[ty * 4 + i];
     if (slot < 0) continue;
     const size_t row = plane_rows > 0 ? (size_t)(slot % top) * plane_rows + slot / top : (size_t)slot;
+    const float os = out_scale != nullptr ? out_scale[slot] : 1.0f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
-      if (n < N) c[row * ldc + n] = from_f32<TC>(acc[i][j]);
+      float v = acc[i][j];
+      if (act == 2) v = v > 0.f ? v * v : 0.f;
+      if (n < N) c[row * ldc + n] = from_f32<TC>(v * os);
     }
   }
 }
@@ -163,7 +199,7 @@ __global__ void __launch_bounds__(256)
 gather_scale_kernel(const uint16_t* __restrict__ x, int ldx, const float* __restrict__ score,
                     const int32_t* __restrict__ perm, uint16_t* __restrict__ xs, int K, int top) {
   const int place = blockIdx.x, slot = perm[place];
-  const float sc = score[slot];
+  const float sc = score != nullptr ? score[slot] : 1.0f;      // (no scores: the inputs as they are)
   const uint16_t* src = x + (size_t)(slot / top) * ldx;
   for (int k = threadIdx.x; k < K; k += 256) xs[(size_t)place * K + k] = f32_to_bf16_bits(bf16_bits_to_f32(src[k]) * sc);
 }
@@ -172,11 +208,15 @@ gather_scale_kernel(const uint16_t* __restrict__ x, int ldx, const float* __rest
 // NS: blocks of 16 rows of the weight a wave takes.  KSUB: pieces of 32 columns of K a step (2, or 4 for tiles of 64
 // places: a decode step's tile holds a place or two, the product streams the weight, and what it needs is many bytes
 // in flight a step).
-template <bool SWIGLU, int TM, int NS, int KSUB>
+// ACT: 0 the float32 result (times out_scale[slot] where given) by place or by slot; 1 silu(gate) * up over interleaved
+// rows, bfloat16 [places, N / 2]; 2 relu^2 of the result, bfloat16 [places, N].
+template <int ACT, int TM, int NS, int KSUB>
 __global__ void __launch_bounds__(256)
 expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ w, void* __restrict__ c, int ldc,
                         int N, int K, const int32_t* __restrict__ perm, const int32_t* __restrict__ offsets,
-                        const int32_t* __restrict__ tiles, int top, int plane_rows) {
+                        const int32_t* __restrict__ tiles, int top, int plane_rows,
+                        const float* __restrict__ out_scale) {
+  constexpr bool SWIGLU = ACT == 1;
   constexpr int MS = TM / 16;          // blocks of 16 places a tile
   constexpr int KSTEP = 32 * KSUB;     // columns of K a step
   constexpr int kLdsRow = KSTEP + 8;   // bfloat16 elements a row of the activations' tile takes in LDS (padded)
@@ -272,19 +312,64 @@ expert_gemm_mfma_kernel(const uint16_t* __restrict__ a, const uint16_t* __restri
           }
         }
       }
+    } else if constexpr (ACT == 2) {
+#pragma unroll
+      for (int s = 0; s < NS; ++s) {
+        const int n0 = n_base + s * 16 + kg * 4;
+        uint16_t* dst = (uint16_t*)c + (size_t)place * ldc + n0;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float v = acc[s][m][i];
+          if (n0 + i < N) dst[i] = f32_to_bf16_bits(v > 0.f ? v * v : 0.f);
+        }
+      }
     } else {
       const int slot = perm[place];
       const size_t row = plane_rows > 0 ? (size_t)(slot % top) * plane_rows + slot / top : (size_t)place;
+      const float os = out_scale != nullptr ? out_scale[slot] : 1.0f;
 #pragma unroll
       for (int s = 0; s < NS; ++s) {
         const int n0 = n_base + s * 16 + kg * 4;
         float* dst = (float*)c + row * ldc + n0;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (n0 + i < N) dst[i] = acc[s][m][i];
+          if (n0 + i < N) dst[i] = acc[s][m][i] * os;
       }
     }
   }
+}
+
+// out[t, i] = relu(u[t, i])^2 * sigmoid(u[t, off_gate]) for an expert that every token uses: its first product's
+// result u [T, ld] holds the ff columns of the expert and, at off_gate, the token's gate (off_gate < 0: no gate).
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256)
+relu2_gate_kernel(const TI* __restrict__ u, int ld, TO* __restrict__ out, int ff, int off_gate) {
+  const size_t t = blockIdx.x;
+  const float g = off_gate >= 0 ? 1.0f / (1.0f + expf(-to_f32(u[t * ld + off_gate]))) : 1.0f;
+  for (int i = threadIdx.x; i < ff; i += 256) {
+    const float v = to_f32(u[t * ld + i]);
+    out[t * ff + i] = from_f32<TO>(v > 0.f ? v * v * g : 0.f);
+  }
+}
+
+extern "C" int atoma_relu2_gate(const void* u, int u_dtype, int ld, void* out, int out_dtype, int n_tokens, int ff,
+                                int off_gate, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (ff <= 0 || ld < ff || off_gate >= ld) return ATOMA_ERR_SHAPE;
+  dim3 grid(n_tokens), block(256);
+  if (u_dtype == kF32 && out_dtype == kF32)
+    hipLaunchKernelGGL((relu2_gate_kernel<float, float>), grid, block, 0, stream, (const float*)u, ld, (float*)out, ff,
+                       off_gate);
+  else if (u_dtype == kF32 && out_dtype == kBF16)
+    hipLaunchKernelGGL((relu2_gate_kernel<float, bf16_t>), grid, block, 0, stream, (const float*)u, ld, (bf16_t*)out,
+                       ff, off_gate);
+  else if (u_dtype == kBF16 && out_dtype == kBF16)
+    hipLaunchKernelGGL((relu2_gate_kernel<bf16_t, bf16_t>), grid, block, 0, stream, (const bf16_t*)u, ld, (bf16_t*)out,
+                       ff, off_gate);
+  else
+    return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
 }
 
 extern "C" int atoma_gather_scale(const void* x, int ldx, const float* score, const int32_t* perm, void* xs, int K,
@@ -297,35 +382,39 @@ extern "C" int atoma_gather_scale(const void* x, int ldx, const float* score, co
   return 0;
 }
 
-// a [places, K] bfloat16 in the order of perm; w [experts, N, K] bfloat16.  swiglu: c bfloat16 [places, N / 2] (ldc),
-// the rows of w in blocks of 16 gate rows and their 16 up rows; else c float32, by place or (plane_rows > 0) by slot
+// a [places, K] bfloat16 in the order of perm; w [experts, N, K] bfloat16.  act 1: c bfloat16 [places, N / 2] (ldc),
+// the rows of w in blocks of 16 gate rows and their 16 up rows; act 2: c bfloat16 [places, N], relu^2; act 0: c
+// float32, by place or (plane_rows > 0) by slot, times out_scale[slot] where given
 extern "C" int atoma_expert_gemm_mfma(const void* a, const void* w, void* c, int ldc, int N, int K, const int32_t* perm,
                                       const int32_t* offsets, const int32_t* tiles, int max_tiles, int top,
-                                      int plane_rows, int swiglu, int tile_m, hipStream_t stream) {
+                                      int plane_rows, int act, int tile_m, const float* out_scale,
+                                      hipStream_t stream) {
   if (max_tiles <= 0 || N <= 0) return 0;
   if (K <= 0 || K % 32 || N % 32 || (tile_m != 64 && tile_m != 128) || top <= 0 || max_tiles > 65535 || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) ||
-      ldc < (swiglu ? N / 2 : N))
+      act < 0 || act > 2 || ldc < (act == 1 ? N / 2 : N) || (act != 0 && (plane_rows > 0 || out_scale != nullptr)))
     return ATOMA_ERR_SHAPE;
   const int ns = 2;      // (four blocks a wave measured slower for tiles of 128 places: 467 against 336 us)
   dim3 grid((N + 64 * ns - 1) / (64 * ns), max_tiles), block(256);
 #define ATOMA_EGM(SW, TM_, NS_, KSUB_)                                                                           \
   hipLaunchKernelGGL((expert_gemm_mfma_kernel<SW, TM_, NS_, KSUB_>), grid, block, 0, stream, (const uint16_t*)a, \
-                     (const uint16_t*)w, c, ldc, N, K, perm, offsets, tiles, top, plane_rows)
-  if (swiglu && tile_m == 64) ATOMA_EGM(true, 64, 2, 4);
-  else if (swiglu) ATOMA_EGM(true, 128, 2, 2);
-  else if (tile_m == 64) ATOMA_EGM(false, 64, 2, 4);
-  else ATOMA_EGM(false, 128, 2, 2);
+                     (const uint16_t*)w, c, ldc, N, K, perm, offsets, tiles, top, plane_rows, out_scale)
+  if (act == 1 && tile_m == 64) ATOMA_EGM(1, 64, 2, 4);
+  else if (act == 1) ATOMA_EGM(1, 128, 2, 2);
+  else if (act == 2 && tile_m == 64) ATOMA_EGM(2, 64, 2, 4);
+  else if (act == 2) ATOMA_EGM(2, 128, 2, 2);
+  else if (tile_m == 64) ATOMA_EGM(0, 64, 2, 4);
+  else ATOMA_EGM(0, 128, 2, 2);
 #undef ATOMA_EGM
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
 
 extern "C" int atoma_route_topk(const float* logits, int ld, int experts, int top, int32_t* ids, float* weights,
-                                int n_tokens, hipStream_t stream) {
+                                int n_tokens, int softmax, const float* correction, float scale, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (experts <= 0 || experts > 1024 || top <= 0 || top > experts || ld < experts) return ATOMA_ERR_SHAPE;
   hipLaunchKernelGGL(route_topk_kernel, dim3((n_tokens + 3) / 4), dim3(256), 0, stream, logits, ld, experts, top, ids,
-                     weights, n_tokens);
+                     weights, n_tokens, softmax, correction, scale);
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
@@ -351,13 +440,14 @@ extern "C" int atoma_route_group(const int32_t* ids, int n_slots, int experts, i
 extern "C" int atoma_expert_gemm(const void* a, int a_dtype, int lda, int a_div, const float* scale, const void* w,
                                  int w_dtype, void* c, int c_dtype, int ldc, int N, int K, const int32_t* perm,
                                  const int32_t* offsets, const int32_t* tiles, int max_tiles, int top, int plane_rows,
-                                 hipStream_t stream) {
+                                 int act, const float* out_scale, hipStream_t stream) {
   if (max_tiles <= 0 || N <= 0) return 0;
-  if (K <= 0 || lda < K || ldc < N || a_div <= 0 || top <= 0 || max_tiles > 65535) return ATOMA_ERR_SHAPE;
+  if (K <= 0 || lda < K || ldc < N || a_div <= 0 || top <= 0 || max_tiles > 65535 || (act != 0 && act != 2))
+    return ATOMA_ERR_SHAPE;
   dim3 grid((N + kTileN - 1) / kTileN, max_tiles), block(256);
 #define ATOMA_EG(TA, TW, TC)                                                                                       \
   hipLaunchKernelGGL((expert_gemm_kernel<TA, TW, TC>), grid, block, 0, stream, (const TA*)a, lda, a_div, scale,     \
-                     (const TW*)w, (TC*)c, ldc, N, K, perm, offsets, tiles, top, plane_rows)
+                     (const TW*)w, (TC*)c, ldc, N, K, perm, offsets, tiles, top, plane_rows, act, out_scale)
   if (a_dtype == kF32 && w_dtype == kF32 && c_dtype == kF32) ATOMA_EG(float, float, float);
   else if (a_dtype == kF32 && w_dtype == kBF16 && c_dtype == kF32) ATOMA_EG(float, bf16_t, float);
   else if (a_dtype == kBF16 && w_dtype == kBF16 && c_dtype == kF32) ATOMA_EG(bf16_t, bf16_t, float);

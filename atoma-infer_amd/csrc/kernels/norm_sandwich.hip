@@ -235,6 +235,80 @@ extern "C" int atoma_add_normed(float* resid, const void* d0, int dtype0, int pl
   return 0;
 }
 
+// The same sum behind a sublayer, for designs whose layers read a weighted average of all earlier layers' results
+// instead of the last one:
+//
+//   X      = resid + d / sqrt(mean(d^2) + eps) * w_post          the layer's result, kept as results[n - 1]
+//   resid  = sum_(j < n) dw[j] * results[j]                       (float32, j ascending; results[0]: the embedding's rows)
+//   out    = resid / sqrt(mean(resid^2) + eps) * w_next           (optional)
+//
+// results is [layers + 1, T, width] float32 and lives for one step.  One workgroup a row, the row in LDS between the
+// passes.
+template <typename TO>
+__global__ void __launch_bounds__(256)
+depth_average_kernel(float* __restrict__ resid, Term a, Term b, int n_terms, const float* __restrict__ w_post,
+                     float* __restrict__ results, size_t result_stride, int n, const float* __restrict__ dw,
+                     const float* __restrict__ w_next, TO* __restrict__ out, int width, float eps_post,
+                     float eps_next) {
+  extern __shared__ float row[];
+  __shared__ float scratch[4];
+  const size_t base = (size_t)blockIdx.x * width;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    float d = term_at(a, base + i);
+    if (n_terms > 1) d += term_at(b, base + i);
+    row[i] = d;
+    ss += d * d;
+  }
+  float inv = 1.0f;
+  if (w_post != nullptr) {
+    ss = block_sum<4>(ss, scratch);
+    inv = 1.0f / sqrtf(ss / (float)width + eps_post);
+  }
+  const float last = dw[n - 1];
+  float ss2 = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float x = resid[base + i] + (w_post != nullptr ? row[i] * inv * w_post[i] : row[i]);
+    results[(size_t)(n - 1) * result_stride + base + i] = x;
+    float y = 0.f;
+    for (int j = 0; j < n - 1; ++j) y += dw[j] * results[(size_t)j * result_stride + base + i];
+    y += last * x;
+    resid[base + i] = y;
+    row[i] = y;
+    ss2 += y * y;
+  }
+  if (out == nullptr) return;
+  ss2 = block_sum<4>(ss2, scratch);
+  const float inv2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
+  for (int i = threadIdx.x; i < width; i += 256) out[base + i] = from_f32<TO>(row[i] * inv2 * w_next[i]);
+}
+
+extern "C" int atoma_depth_average(float* resid, const void* d0, int dtype0, int planes0, size_t stride0, float scale0,
+                                   const void* d1, int dtype1, int planes1, size_t stride1, float scale1,
+                                   const float* w_post, float eps_post, float* results, size_t result_stride, int n,
+                                   const float* dw, const float* w_next, float eps_next, void* out, int out_dtype,
+                                   int n_rows, int width, hipStream_t stream) {
+  if (n_rows <= 0) return 0;
+  if (width <= 0 || width > 16384 || d0 == nullptr || planes0 <= 0 || (d1 != nullptr && planes1 <= 0) || n < 1 ||
+      results == nullptr || dw == nullptr || result_stride < (size_t)n_rows * width)
+    return ATOMA_ERR_SHAPE;
+  if ((dtype0 != kF32 && dtype0 != kBF16) || (d1 != nullptr && dtype1 != kF32 && dtype1 != kBF16)) return ATOMA_ERR_DTYPE;
+  Term a{d0, dtype0, planes0, stride0, scale0}, b{d1, dtype1, planes1, stride1, scale1};
+  const int n_terms = d1 != nullptr ? 2 : 1;
+  const size_t lds = (size_t)width * sizeof(float);
+  dim3 grid(n_rows), block(256);
+  if (out == nullptr || out_dtype == kF32)
+    hipLaunchKernelGGL((depth_average_kernel<float>), grid, block, lds, stream, resid, a, b, n_terms, w_post, results,
+                       result_stride, n, dw, w_next, (float*)out, width, eps_post, eps_next);
+  else if (out_dtype == kBF16)
+    hipLaunchKernelGGL((depth_average_kernel<bf16_t>), grid, block, lds, stream, resid, a, b, n_terms, w_post, results,
+                       result_stride, n, dw, w_next, (bf16_t*)out, width, eps_post, eps_next);
+  else
+    return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
 // Rows of the stream set anew: resid[t] = y[t] + bias (float32), for a map of the whole stream that replaces it
 // (the entry of a pass over looped layers).  The second kernel packs the rows of two float32 streams side by side in
 // the activation dtype, [a | b], as such a map's input.

@@ -54,6 +54,8 @@ HIP_MODULES: Dict[str, Tuple[Sequence[str], Sequence[str]]] = {
     "experts": (("experts.hip",), ()),
     "state_space": (("state_space.hip",), ()),
     "latent": (("latent.hip",), ()),
+    "differential": (("differential.hip",), ()),
+    "mingru": (("mingru.hip",), ()),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

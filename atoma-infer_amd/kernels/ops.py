@@ -240,8 +240,11 @@ def paged_attention_generic(q: torch.Tensor, kcache: torch.Tensor, vcache: torch
         page_size, t, nh, nkv, hd, _p(slopes), int(chunk), _p(sinks), _stream()), "paged_attention_generic")
 
 
-def swiglu(gu: torch.Tensor, out: Optional[torch.Tensor] = None, block: int = 0) -> torch.Tensor:
-    """out[t, i] = silu(gate[t, i]) * up[t, i] for gu [T, 2 I].
+GATE_ACTIVATIONS = {"silu": 0, "gelu_tanh": 1}
+
+
+def swiglu(gu: torch.Tensor, out: Optional[torch.Tensor] = None, block: int = 0, act: str = "silu") -> torch.Tensor:
+    """out[t, i] = act(gate[t, i]) * up[t, i] for gu [T, 2 I]; ``act``: "silu", or "gelu_tanh" (gelu's tanh form).
 
     ``block`` 0: gate is the first half of a row and up the second; 16: blocks of 16 gate values followed by
     their 16 up values (the order of the fused gate-up product's weight rows).
@@ -252,7 +255,8 @@ def swiglu(gu: torch.Tensor, out: Optional[torch.Tensor] = None, block: int = 0)
     if out is None:
         out = torch.empty((t, inter), dtype=gu.dtype, device=gu.device)
     _need(out.is_contiguous() and tuple(out.shape) == (t, inter) and out.dtype is gu.dtype, "swiglu: bad out")
-    _check(core().atoma_swiglu(_p(gu), _p(out), _code(gu, "swiglu input"), t, inter, int(block), _stream()), "swiglu")
+    _check(core().atoma_swiglu(_p(gu), _p(out), _code(gu, "swiglu input"), t, inter, int(block),
+                               GATE_ACTIVATIONS[act], _stream()), "swiglu")
     return out
 
 
@@ -647,14 +651,21 @@ def head_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gate: 
 
 
 
-def route_topk(logits: torch.Tensor, top: int):
-    """(ids int32 [T, top], scores float32 [T, top]): the ``top`` largest sigmoid(logits) of each row."""
-    _dev(logits)
+def route_topk(logits: torch.Tensor, top: int, score: str = "sigmoid", correction: Optional[torch.Tensor] = None,
+               scale: float = 1.0):
+    """(ids int32 [T, top], weights float32 [T, top]).  Scores are sigmoid(logits) or ("softmax") the softmax of a
+    row; the ``top`` experts with the largest score + ``correction`` [experts] are chosen and weighed by
+    score * ``scale``."""
+    _dev(logits, correction)
+    _need(score in ("sigmoid", "softmax"), "route_topk: scores are 'sigmoid' or 'softmax'")
+    if correction is not None:
+        _f32(correction, "correction", logits.shape[1])
     _need(logits.dtype is torch.float32 and logits.dim() == 2 and logits.stride(1) == 1, "router logits: float32 [T, E]")
     t, e = logits.shape
     ids = torch.empty((t, top), dtype=torch.int32, device=logits.device)
     scores = torch.empty((t, top), dtype=torch.float32, device=logits.device)
     _check(_module("experts").atoma_route_topk(_p(logits), logits.stride(0), e, int(top), _p(ids), _p(scores), t,
+                                               1 if score == "softmax" else 0, _p(correction), ctypes.c_float(scale),
                                                _stream()), "route_topk")
     return ids, scores
 
@@ -676,11 +687,15 @@ def route_group(ids: torch.Tensor, experts: int, tile_m: int = 64):
 
 
 def expert_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, perm, offsets, tiles, top: int, *,
-                gather: bool, scale: Optional[torch.Tensor] = None, planes: bool = False) -> None:
+                gather: bool, scale: Optional[torch.Tensor] = None, planes: bool = False, relu2: bool = False,
+                out_scale: Optional[torch.Tensor] = None) -> None:
     """out[row(slot)] = (scale[slot] * a[src(slot)]) @ w[expert(slot)]^T in float32 arithmetic, for every slot.
     ``gather``: src is the slot's token (a [T, K]), else the slot (a [slots, K]).  ``planes``: out is [top, T, N]
-    and choice c of token t goes to out[c, t], else out is [slots, N]."""
-    _dev(a, w, out, perm, offsets, tiles, scale)
+    and choice c of token t goes to out[c, t], else out is [slots, N].  ``relu2``: the result's positive part squared;
+    ``out_scale`` [slots] multiplies the result."""
+    _dev(a, w, out, perm, offsets, tiles, scale, out_scale)
+    if out_scale is not None:
+        _f32(out_scale, "out_scale", perm.numel())
     n_slots = perm.numel()
     e, n, k = w.shape
     _need(w.is_contiguous() and a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k, "expert_gemm: a and w do not fit")
@@ -692,15 +707,17 @@ def expert_gemm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, perm, offse
     _check(_module("experts").atoma_expert_gemm(
         _p(a), _code(a, "a"), a.stride(0) if a.shape[0] > 1 else k, top if gather else 1, _p(scale), _p(w),
         _code(w, "w"), _p(out), _code(out, "out"), n, n, k, _p(perm), _p(offsets), _p(tiles), tiles.shape[0], int(top),
-        n_slots // top if planes else 0, _stream()), "expert_gemm")
+        n_slots // top if planes else 0, 2 if relu2 else 0, _p(out_scale), _stream()), "expert_gemm")
 
 
-def gather_scale(x: torch.Tensor, scores: torch.Tensor, perm: torch.Tensor, top: int) -> torch.Tensor:
-    """xs[place] = bfloat16(scores[slot] * x[slot // top]) for slot = perm[place]: the experts' inputs in their order."""
+def gather_scale(x: torch.Tensor, scores: Optional[torch.Tensor], perm: torch.Tensor, top: int) -> torch.Tensor:
+    """xs[place] = bfloat16(scores[slot] * x[slot // top]) for slot = perm[place]: the experts' inputs in their order
+    (without ``scores``: the inputs as they are)."""
     _dev(x, scores, perm)
     n, k = perm.numel(), x.shape[1]
     _need(x.dtype is torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.shape[0] * top == n, "gather_scale: bad x")
-    _f32(scores, "scores", n)
+    if scores is not None:
+        _f32(scores, "scores", n)
     _i32(perm, "perm", n)
     xs = torch.empty((n, k), dtype=torch.bfloat16, device=x.device)
     _check(_module("experts").atoma_gather_scale(_p(x), x.stride(0) if x.shape[0] > 1 else k, _p(scores), _p(perm),
@@ -713,24 +730,181 @@ def expert_gemm_mfma_ok(n: int, k: int) -> bool:
 
 
 def expert_gemm_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, perm, offsets, tiles, top: int, *,
-                     swiglu: bool = False, planes: bool = False, tile_m: int = 64) -> None:
+                     swiglu: bool = False, planes: bool = False, tile_m: int = 64, relu2: bool = False,
+                     out_scale: Optional[torch.Tensor] = None) -> None:
     """The grouped product on the matrix cores: a bfloat16 [places, K] in the order of ``perm``, w bfloat16
     [experts, N, K].  ``swiglu``: w's rows in blocks of 16 gate rows and their 16 up rows, out bfloat16
-    [places, N / 2] = silu(gate) * up; else out float32 [places, N] or, with ``planes``, [top, T, N] by slot.
+    [places, N / 2] = silu(gate) * up; ``relu2``: out bfloat16 [places, N], the result's positive part squared; else out
+    float32 [places, N] or, with ``planes``, [top, T, N] by slot, times ``out_scale`` [slots] where given.
     ``tile_m``: what ``route_group`` was told."""
-    _dev(a, w, out, perm, offsets, tiles)
+    _dev(a, w, out, perm, offsets, tiles, out_scale)
+    _need(not (swiglu and relu2), "expert_gemm_mfma: one activation")
+    if out_scale is not None:
+        _f32(out_scale, "out_scale", perm.numel())
     n_slots = perm.numel()
     e, n, k = w.shape
     _need(a.dtype is torch.bfloat16 and w.dtype is torch.bfloat16 and a.is_contiguous() and w.is_contiguous()
           and tuple(a.shape) == (n_slots, k) and expert_gemm_mfma_ok(n, k), "expert_gemm_mfma: operands do not fit")
     cols = n // 2 if swiglu else n
     _need(out.is_contiguous() and out.numel() == n_slots * cols and out.shape[-1] == cols
-          and out.dtype is (torch.bfloat16 if swiglu else torch.float32) and not (swiglu and planes),
-          "expert_gemm_mfma: bad out")
+          and out.dtype is (torch.bfloat16 if swiglu or relu2 else torch.float32)
+          and not ((swiglu or relu2) and (planes or out_scale is not None)), "expert_gemm_mfma: bad out")
     _need(offsets.numel() == e + 1 and tiles.dim() == 2 and tiles.shape[1] == 2, "expert_gemm_mfma: bad grouping")
     _check(_module("experts").atoma_expert_gemm_mfma(
         _p(a), _p(w), _p(out), cols, n, k, _p(perm), _p(offsets), _p(tiles), tiles.shape[0], int(top),
-        n_slots // top if planes else 0, 1 if swiglu else 0, int(tile_m), _stream()), "expert_gemm_mfma")
+        n_slots // top if planes else 0, 1 if swiglu else 2 if relu2 else 0, int(tile_m), _p(out_scale), _stream()),
+        "expert_gemm_mfma")
+
+
+def relu2_gate(u: torch.Tensor, ff: int, off_gate: int, out_dtype: torch.dtype) -> torch.Tensor:
+    """out[t, i] = relu(u[t, i])^2 * sigmoid(u[t, off_gate]) for i < ff (``off_gate`` < 0: no gate), u [T, >= ff]."""
+    _dev(u)
+    _need(u.dim() == 2 and u.stride(1) == 1 and u.shape[1] >= ff and off_gate < u.shape[1], "relu2_gate: bad input")
+    t = u.shape[0]
+    out = torch.empty((t, ff), dtype=out_dtype, device=u.device)
+    _check(_module("experts").atoma_relu2_gate(_p(u), _code(u, "u"), u.stride(0) if t > 1 else u.shape[1], _p(out),
+                                               _code(out, "out"), t, int(ff), int(off_gate), _stream()), "relu2_gate")
+    return out
+
+
+def depth_average(resid: torch.Tensor, terms, w_post: Optional[torch.Tensor], eps_post: float, results: torch.Tensor,
+                  n: int, weights: torch.Tensor, w_next: Optional[torch.Tensor] = None, eps_next: float = 0.0,
+                  out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """X = resid + rmsnorm(sum_i scale_i * term_i) * w_post is kept as results[n - 1]; resid becomes
+    sum_(j < n) weights[j] * results[j] (float32); with ``w_next`` also returns rmsnorm(resid) * w_next in
+    ``out_dtype``.  ``results``: float32 [>= n, T, W]; ``terms`` as for ``add_normed``."""
+    _need(resid.dtype is torch.float32 and resid.dim() == 2 and resid.is_contiguous(), "resid must be float32 [T, W]")
+    t, width = resid.shape
+    _need(1 <= len(terms) <= 2, "one or two terms")
+    _need(width <= 16000, "rows of more than 16,000 columns do not fit the kernel's row buffer")
+    _dev(resid, w_post, w_next, results, weights, *[d for d, _ in terms])
+    _need(results.dtype is torch.float32 and results.dim() == 3 and results.is_contiguous()
+          and tuple(results.shape[1:]) == (t, width) and 1 <= n <= results.shape[0], "depth_average: bad results")
+    _f32(weights, "depth weights", n)
+    if w_post is not None:
+        _f32(w_post, "norm weight", width)
+    out = None
+    if w_next is not None:
+        _f32(w_next, "norm weight", width)
+        out = torch.empty((t, width), dtype=out_dtype, device=resid.device)
+    a = _term(terms[0][0], t, width)
+    b = _term(terms[1][0], t, width) if len(terms) > 1 else (_p(None), F32, 0, ctypes.c_size_t(0))
+    _check(_module("layer_norms").atoma_depth_average(
+        _p(resid), *a, ctypes.c_float(terms[0][1]), *b, ctypes.c_float(terms[1][1] if len(terms) > 1 else 0.0),
+        _p(w_post), ctypes.c_float(eps_post), _p(results), ctypes.c_size_t(t * width), int(n), _p(weights), _p(w_next),
+        ctypes.c_float(eps_next), _p(out), _code(out, "out") if out is not None else F32, t, width, _stream()),
+        "depth_average")
+    return out
+
+
+def diff_prepare(proj: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor, rot_dim: int, q_out: torch.Tensor,
+                 kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], slot_mapping: Optional[torch.Tensor],
+                 page_size: int, heads: int, kv_heads: int, dim: int, vdim: int, hdo: int, offsets) -> torch.Tensor:
+    """Differential attention's inputs from the fused projection [q | k | v | g] (see differential.hip): rotated
+    queries to ``q_out`` [T, 2 heads, hdo], keys [k1 | k2 | 0] and values [v | 0] into their tiles, and the heads'
+    gates, sigmoid applied, as float32 [T, heads] (returned).  ``offsets`` = (k, v, g) columns of ``proj``; without
+    tiles ``proj`` needs q and g only."""
+    _dev(proj, positions, inv_freq, q_out, kcache, vcache, slot_mapping)
+    t = proj.shape[0]
+    off_k, off_v, off_g = (int(o) for o in offsets)
+    _need(proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= off_g + heads, "diff_prepare: bad projection")
+    _need(2 * heads * dim <= min(off_g, off_k if kcache is not None else off_g), "diff_prepare: offsets overlap q")
+    _i32(positions, "positions", t)
+    _f32(inv_freq, "inv_freq", rot_dim // 2)
+    _need(q_out.dim() == 2 and q_out.is_contiguous() and tuple(q_out.shape) == (t, 2 * heads * hdo), "diff_prepare: bad q_out")
+    cache_code = _code(q_out, "q_out")
+    if kcache is not None:
+        _need(slot_mapping is not None and vcache is not None, "a cache write needs slots and both tiles")
+        _i32(slot_mapping, "slot_mapping", t)
+        _need(off_k + 2 * kv_heads * dim <= off_v and off_v + kv_heads * vdim <= off_g, "diff_prepare: offsets overlap")
+        pages = kcache.shape[0]
+        _need(kcache.is_contiguous() and tuple(kcache.shape) == (pages, kv_heads, page_size * hdo)
+              and vcache.is_contiguous() and tuple(vcache.shape) == tuple(kcache.shape)
+              and vcache.dtype is kcache.dtype, "diff_prepare: the tiles must be [pages, kv_heads, page_size * hdo]")
+        cache_code = _code(kcache, "cache")
+    gate = torch.empty((t, heads), dtype=torch.float32, device=proj.device)
+    _check(_module("differential").atoma_diff_prepare(
+        _p(proj), _code(proj, "proj"), proj.stride(0) if t > 1 else proj.shape[1], _p(positions), _p(inv_freq),
+        int(rot_dim), _p(q_out), q_out.stride(0), _code(q_out, "q_out"), _p(kcache), _p(vcache), cache_code,
+        _p(slot_mapping), int(page_size), _p(gate), t, heads, kv_heads, dim, vdim, hdo, off_k, off_v, off_g, _stream()),
+        "diff_prepare")
+    return gate
+
+
+def diff_combine(att: torch.Tensor, gate: torch.Tensor, heads: int, vdim: int, hdo: int, lam: float, eps: float,
+                 post: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """y[t, h] = (a1 - lam a2) / sqrt(mean((a1 - lam a2)^2) + eps) * post * gate[t, h] over the first ``vdim`` columns
+    of the two maps' outputs att[t, 2h] and att[t, 2h + 1] ([T, 2 heads * hdo]); y [T, heads * vdim]."""
+    _dev(att, gate)
+    t = att.shape[0]
+    _need(att.dim() == 2 and att.is_contiguous() and att.shape[1] == 2 * heads * hdo, "diff_combine: bad input")
+    _f32(gate, "gate", t * heads)
+    y = torch.empty((t, heads * vdim), dtype=out_dtype, device=att.device)
+    _check(_module("differential").atoma_diff_combine(
+        _p(att), _code(att, "att"), att.shape[1], _p(gate), _p(y), _code(y, "y"), heads * vdim, t, heads, vdim, hdo,
+        ctypes.c_float(lam), ctypes.c_float(eps), ctypes.c_float(post), _stream()), "diff_combine")
+    return y
+
+
+MINGRU_STRETCH_MIN_TOKENS = 64      # entries of at least this many tokens are walked in stretches side by side
+
+
+def mingru_plan(counts, width: int, compute_units: int = 256):
+    """The stretches of a step for ``mingru``: int32 [n][3] of (entry, first token, end) followed by [entries + 1] of
+    each entry's first stretch; None when no entry is long enough to pay for it.  A function of the entries' lengths."""
+    import numpy as np
+    counts = np.asarray(counts, dtype=np.int64)
+    if counts.size == 0 or int(counts.max()) < MINGRU_STRETCH_MIN_TOKENS:
+        return None
+    # stretches long enough to amortise the second read of their tokens, short enough that the step's stretches
+    # times the channels' workgroups give every compute unit a few workgroups
+    blocks = -(-width // 256)
+    total = int(counts.sum())
+    length = max(16, min(256, (total * blocks) // (4 * compute_units)))
+    rows, first, t0 = [], [0], 0
+    for e, c in enumerate(counts.tolist()):
+        for lo in range(0, c, length):
+            rows.append((e, t0 + lo, t0 + min(lo + length, c)))
+        first.append(len(rows))
+        t0 += c
+    if len(rows) > 65535:
+        return None
+    return np.concatenate([np.asarray(rows, dtype=np.int32).reshape(-1), np.asarray(first, dtype=np.int32)]), len(rows)
+
+
+def mingru(proj: torch.Tensor, off_x: int, off_g: int, width: int, bz: torch.Tensor, bx: torch.Tensor,
+           q_start: torch.Tensor, state_slots: torch.Tensor, state: torch.Tensor, out_dtype: torch.dtype,
+           plan=None) -> torch.Tensor:
+    """The minGRU recurrence over a step's entries (see mingru.hip): proj float32 [T, >= off_g + width] holds the
+    columns of z (from 0), x and g; y [T, width] = S * silu(g) with each request's S [width] read from and written to
+    its row of ``state``.  ``plan``: (int32 device tensor, stretches) from ``mingru_plan``, or None for the plain walk."""
+    _dev(proj, bz, bx, q_start, state_slots, state)
+    t = proj.shape[0]
+    n_entries = state_slots.numel()
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= off_g + width
+          and off_x >= width and off_g >= off_x + width, "mingru: bad projection")
+    _f32(bz, "z bias", width)
+    _f32(bx, "x bias", width)
+    _i32(q_start, "q_start", n_entries + 1)
+    _i32(state_slots, "state_slots")
+    _need(state.dtype is torch.float32 and state.is_contiguous() and state.dim() == 2 and state.shape[1] == width,
+          "mingru: the state must be float32 [slots, width]")
+    y = torch.empty((t, width), dtype=out_dtype, device=proj.device)
+    ld = proj.stride(0) if t > 1 else proj.shape[1]
+    lib = _module("mingru")
+    if plan is None or plan[1] == 0:
+        _check(lib.atoma_mingru_scan(_p(proj), ld, _p(bz), _p(bx), _p(q_start), _p(state_slots), _p(state), _p(y),
+                                     _code(y, "y"), width, n_entries, width, int(off_x), int(off_g), _stream()),
+               "mingru_scan")
+        return y
+    arr, n_st = plan
+    _i32(arr, "stretches", 3 * n_st + n_entries + 1)
+    ab = torch.empty((n_st, 2, width), dtype=torch.float32, device=proj.device)
+    first = ctypes.c_void_p(arr.data_ptr() + 12 * n_st)
+    _check(lib.atoma_mingru_stretched(_p(proj), ld, _p(bz), _p(bx), _p(arr), int(n_st), first, _p(state_slots),
+                                      _p(state), _p(ab), _p(y), _code(y, "y"), width, n_entries, width, int(off_x),
+                                      int(off_g), _stream()), "mingru_stretched")
+    return y
 
 
 SPLIT_MAX_VOCAB = 262144       # the largest vocabulary whose rows ``sample_packed(split=True)`` cuts into parts

@@ -53,6 +53,11 @@ class Model:
         # stream's own rows are summed into in place), and one that is run several times is told which run this is
         embedded = spec.embedding[1].forward(ctx.tokens) if any(getattr(b, "reads_embedding", False) for b in blocks) \
             else None
+        # blocks that weigh the results of all blocks before them: the results of one step, the embedding's rows first
+        results = None
+        if any(getattr(b, "keeps_results", False) for b in blocks):
+            results = torch.empty((len(blocks) + 1, *resid.shape), dtype=torch.float32, device=resid.device)
+            spec.embedding[1].forward(ctx.tokens, out=results[0])
         runs = {}
         for pos, block in enumerate(blocks):
             extra = {}
@@ -60,6 +65,8 @@ class Model:
                 extra["next_norm"] = readers[pos]
             if getattr(block, "reads_embedding", False):
                 extra["embedded"] = embedded
+            if getattr(block, "keeps_results", False):
+                extra["results"], extra["position"] = results, pos
             if getattr(block, "takes_turn", False):
                 layer = spec.run_order[pos].layer
                 extra["turn"] = runs.get(layer, 0)

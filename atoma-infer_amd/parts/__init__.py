@@ -2,8 +2,8 @@
 from .base import (Block, CacheSpec, FeedForward, Mixer, Norm, Part, PositionEncoding, StateSpec, WeightSpec,
                    make_part, register_block, register_feed_forward, register_mixer, register_norm,
                    register_position, registered_kinds)
-from .attention import LatentAttention, PagedAttention, TiedValueAttention
-from .block import PreNormBlock, SandwichBlock, SideBySideBlock
+from .attention import DifferentialAttention, LatentAttention, PagedAttention, TiedValueAttention
+from .block import DepthAverage, PreNormBlock, SandwichBlock, SideBySideBlock
 from .loop import LoopEntry, NoMixer
 from .embedding import OutputHead, TokenEmbedding
 from .experts import RoutedExperts
@@ -12,11 +12,11 @@ from .linear import linear
 from .norm import RMSNorm
 from .parallel import ParallelMixer
 from .position import NoPosition, RotaryEncoding
-from .recurrent import GatedDeltaRule, StateSpaceDuality
+from .recurrent import GatedDeltaRule, MinGRU, StateSpaceDuality
 
 __all__ = ["Block", "CacheSpec", "FeedForward", "Mixer", "Norm", "Part", "PositionEncoding", "StateSpec",
            "WeightSpec", "make_part", "register_block", "register_feed_forward", "register_mixer", "register_norm",
            "register_position", "registered_kinds", "PagedAttention", "PreNormBlock", "OutputHead",
            "TokenEmbedding", "SwiGLU", "linear", "RMSNorm", "NoPosition", "RotaryEncoding", "TiedValueAttention",
            "SandwichBlock", "RoutedExperts", "ParallelMixer", "GatedDeltaRule", "LatentAttention", "SideBySideBlock",
-           "LoopEntry", "NoMixer", "StateSpaceDuality"]
+           "LoopEntry", "NoMixer", "StateSpaceDuality", "DifferentialAttention", "MinGRU", "DepthAverage"]

@@ -379,6 +379,117 @@ class LatentAttention(PagedAttention):
         return linear_delta(out, self.w_o, sink, self.w_o_tiled)
 
 
+class DifferentialAttention(PagedAttention):
+    """Attention whose heads each hold two score maps over one set of values and put out the difference of the two
+    attentions:
+
+    * q = W_q x has ``heads`` x 2 maps of ``head_size`` columns, k = W_k x has ``kv_heads`` x 2, laid out head by head
+      as [map 1 | map 2]; v = W_v x has ``kv_heads`` heads of ``value_size``; query head h reads key/value head
+      h // (heads / kv_heads);
+    * the first ``rotary_dim`` columns of every map of q and k are turned in half-split pairs (c, c + rotary_dim / 2)
+      by position * rotary_base^(-2c / rotary_dim) / ``rotary_factor``; angles are worked out in float32 from the
+      position, so there is no table and no largest position;
+    * each map is a causal softmax attention a1, a2 with the scale given; o = a1 - lam a2 with
+      lam = exp(lq1 . lk1) - exp(lq2 . lk2) + ``diff`` (one number a layer, from four small tensors); o is divided by
+      its root mean square over the head's values (eps inside the root, no weight), multiplied by 1 - ``diff`` and
+      by sigmoid(W_g x)_head; then W_o.
+
+    How it runs: a key/value head of the cache keeps [k1 | k2] as ONE key of 2 head_size columns and v once, and the
+    two maps of a query head are two query heads of that width, map m holding its columns at m * head_size and
+    zeros elsewhere, so q' . k' = q_m . k_m.  The framework's attention kernels (matrix-core and general) then serve
+    with 2 heads query heads over kv_heads key heads; ``self.hd`` is max(2 head_size, value_size) as a multiple of 16.
+    A call that reads another call's cache (``kv_from``) has no k and v tensors and projects q and g only.
+
+    Tensors ([out, in]): ``q``, ``k``, ``v``, ``g`` [heads, width], ``o`` [width, heads * value_size], ``lq1``,
+    ``lk1``, ``lq2``, ``lk2`` [head_size].
+    """
+
+    def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_size: int, value_size: int, scale: float,
+                 diff: float, norm_eps: float, rotary_base: float = 10000.0, rotary_dim: int = 0,
+                 rotary_factor: float = 1.0, owns_cache: bool = True):
+        wide = -(-max(2 * int(head_size), int(value_size)) // 16) * 16
+        if num_heads % num_kv_heads:
+            raise ValueError(f"{num_heads} query heads cannot be grouped over {num_kv_heads} KV heads")
+        super().__init__(width, 2 * num_heads, num_kv_heads, wide, None, None, scale, None)
+        if rotary_dim % 2 or not 0 <= rotary_dim <= head_size or rotary_dim > 256:
+            raise ValueError(f"rotary_dim {rotary_dim} must be even, at most the head size {head_size} and at most 256")
+        if value_size > 256:
+            raise ValueError("values of more than 256 columns a head are not supported")
+        self.heads, self.dim, self.vdim = int(num_heads), int(head_size), int(value_size)
+        self.hd_in = self.vd_in = wide
+        self.diff, self.norm_eps = float(diff), float(norm_eps)
+        self.rotary_base, self.rotary_dim, self.rotary_factor = float(rotary_base), int(rotary_dim), float(rotary_factor)
+        if not self.rotary_factor > 0:
+            raise ValueError("the rotation's scaling factor must be positive")
+        self.owns_cache = bool(owns_cache)
+        nq = 2 * self.heads * self.dim
+        # columns of the fused projection: q, then (with a cache of its own) k and v, then the heads' gates
+        self.off_k = nq
+        self.off_v = nq + 2 * self.nkv * self.dim
+        self.off_g = self.off_v + self.nkv * self.vdim if self.owns_cache else nq
+        self.w_in = self.inv_freq = None
+        self.lam = 0.0
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, g, d, v, w = self.heads, self.nkv, self.dim, self.vdim, self.width
+        specs = {"q": WeightSpec((h * 2 * d, w))}
+        if self.owns_cache:
+            specs.update({"k": WeightSpec((g * 2 * d, w)), "v": WeightSpec((g * v, w))})
+        specs.update({"lq1": WeightSpec((d,), std=0.1), "lk1": WeightSpec((d,), std=0.1),
+                      "lq2": WeightSpec((d,), std=0.1), "lk2": WeightSpec((d,), std=0.1),
+                      "g": WeightSpec((h, w), std=0.1), "o": WeightSpec((w, h * v))})
+        return specs
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("q")] + ([get("k"), get("v")] if self.owns_cache else []) + [get("g")]
+        dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        rows = sum(w.shape[0] for w in ws)
+        parts = [w.to(device=device, dtype=dt) for w in ws]
+        if (-rows) % 64:      # whole tiles for the matrix-core products
+            parts.append(torch.zeros(((-rows) % 64, self.width), dtype=dt, device=device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        # one number a layer, worked out once in float32 as the design asks of everything around the scores
+        f32 = lambda n: get(n).to(torch.float32)
+        self.lam = float(torch.exp((f32("lq1") * f32("lk1")).sum()) - torch.exp((f32("lq2") * f32("lk2")).sum())
+                         + torch.tensor(self.diff, dtype=torch.float32))
+        # base^(-2c / dims) / factor in double precision, rounded once to float32
+        c = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+        freq = torch.pow(torch.tensor(self.rotary_base, dtype=torch.float64), -2.0 * c / max(self.rotary_dim, 1))
+        self.inv_freq = (freq / self.rotary_factor).to(device=device, dtype=torch.float32).contiguous()
+        self.act_dtype = act_dtype
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_o))
+
+    accepts_begun = False
+    takes_sink = False
+
+    def forward(self, x, ctx, cache, sink=None):
+        if cache.writable != self.owns_cache:
+            raise RuntimeError("differential attention: a layer with k and v tensors writes its own cache, one "
+                               "without reads another layer's")
+        t = x.shape[0]
+        # the projection leaves in float32: rotation and gates are float32 work
+        proj = linear(x, self.w_in, torch.float32)
+        q = torch.empty((t, self.nh * self.hd), dtype=x.dtype, device=x.device)
+        k, v, slots = (cache.k, cache.v, cache.slot_mapping) if self.owns_cache else (None, None, None)
+        gate = ops.diff_prepare(proj, ctx.positions, self.inv_freq, self.rotary_dim, q, k, v, slots, cache.page_size,
+                                self.heads, self.nkv, self.dim, self.vdim, self.hd, (self.off_k, self.off_v, self.off_g))
+        att = torch.empty((t, self.nh * self.hd), dtype=x.dtype, device=x.device)
+        self.attend(q, cache.k, cache.v, att, ctx, cache)
+        y = ops.diff_combine(att, gate, self.heads, self.vdim, self.hd, self.lam, self.norm_eps, 1.0 - self.diff, x.dtype)
+        return linear_delta(y, self.w_o, None, self.w_o_tiled)
+
+
 register_mixer("latent_attention", LatentAttention)
+register_mixer("differential_attention", DifferentialAttention)
 register_mixer("attention", PagedAttention)
 register_mixer("tied_value_attention", TiedValueAttention)

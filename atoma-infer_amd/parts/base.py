@@ -237,6 +237,10 @@ class Block(Part):
     fuses_next_norm = False
     #: True if ``forward`` has a keyword ``embedded``: the float32 rows as the embedding left them
     reads_embedding = False
+    #: True if ``forward`` has keywords ``results`` and ``position``: a float32 tensor [blocks + 1, T, width] that lives
+    #: for one step, whose row 0 holds the embedding's rows and row j + 1 is the block at run-order position j's to
+    #: fill with its result, and this call's position in the run order
+    keeps_results = False
     #: True if ``forward`` has a keyword ``turn``: how many calls of this block the run order has before this one
     takes_turn = False
 

@@ -9,7 +9,8 @@ two outputs travel on unsummed, and the kernel of the norm that reads the stream
 
 ``SandwichBlock``: a norm before and a norm behind each sublayer, ``h = x + norm1b(mixer(norm1(x)))``,
 ``y = h + norm2b(ffn(norm2(h)))``; the feed-forward half may be absent.  One kernel norms a sublayer's output, adds
-it to the stream and applies the norm that reads the stream next.
+it to the stream and applies the norm that reads the stream next.  With a ``DepthAverage`` the block's result y is
+kept beside those of all blocks before it, and what the stream carries on is a weighted sum of them all.
 """
 from __future__ import annotations
 
@@ -18,7 +19,7 @@ from typing import Dict, Optional
 import torch
 
 from ..kernels import ops
-from .base import Begun, Block, FeedForward, Mixer, Norm, WeightSpec, register_block
+from .base import Begun, Block, FeedForward, Mixer, Norm, Part, WeightSpec, register_block
 from .linear import Normed, ResidualSink
 
 BEGUN_ROWS = 16      # rows of a step up to which products begin and finish norms (kernels.gemm_bf16.BEGUN_MAX_M)
@@ -81,21 +82,47 @@ def _join(prefix: str, rel: str) -> str:
     return f"{prefix}.{rel}" if prefix and rel else prefix or rel
 
 
+class DepthAverage(Part):
+    """The weights of a block that hands on, instead of its own result, a weighted sum of the results of all blocks
+    up to itself: with X_0 the embedding's rows and X_(j+1) the result of the block at run-order position j, the
+    block at position i leaves ``sum_(j <= i + 1) w[j] X_j`` in the stream.  ``count`` = i + 2 weights, one tensor
+    (``name``), kept and applied in float32."""
+
+    def __init__(self, count: int, name: str = "dwa"):
+        if count < 2:
+            raise ValueError("a depth average has at least the embedding's rows and one block's result to weigh")
+        self.count, self.name = int(count), str(name)
+        self.weights: Optional[torch.Tensor] = None
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {self.name: WeightSpec((self.count,), "tail_heavy", mean=0.3 / self.count, std=0.05)}
+
+    def load(self, get, device, act_dtype) -> None:
+        self.weights = get(self.name).to(device=device, dtype=torch.float32).contiguous()
+
+
 class SandwichBlock(Block):
     """``norms`` = (before the mixer, behind it, before the feed-forward, behind it); the last two and the
     feed-forward are None for a layer that has the mixer only.  ``names``: the children's prefixes below the
-    layer's, in the order (norms..., mixer, feed-forward); a norm whose tensor carries its whole name has prefix ""."""
+    layer's, in the order (norms..., mixer, feed-forward, depth average); a part whose tensor carries its whole name
+    has prefix "".  ``depth_average``: see ``DepthAverage``; the model then hands ``forward`` the results kept so far
+    (``keeps_results``)."""
 
     def __init__(self, norms, mixer: Mixer, feed_forward: Optional[FeedForward] = None,
-                 names=("", "", "", "", "mix", "mlp")):
+                 names=("", "", "", "", "mix", "mlp", ""), depth_average: Optional[DepthAverage] = None):
         self.norm1, self.norm1b, self.norm2, self.norm2b = norms
         self.mixer, self.feed_forward = mixer, feed_forward
         if (feed_forward is None) != (self.norm2 is None) or (feed_forward is None) != (self.norm2b is None):
             raise ValueError("the feed-forward and its two norms come together or not at all")
-        self.names = tuple(names)
+        self.names = tuple(names) + ("",) * (7 - len(names))
+        self.depth_average = depth_average
+        self.keeps_results = depth_average is not None
 
     def _children(self):
-        parts = (self.norm1, self.norm1b, self.norm2, self.norm2b, self.mixer, self.feed_forward)
+        parts = (self.norm1, self.norm1b, self.norm2, self.norm2b, self.mixer, self.feed_forward, self.depth_average)
         return [(n, p) for n, p in zip(self.names, parts) if p is not None]
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
@@ -116,7 +143,7 @@ class SandwichBlock(Block):
     def entry_norm(self):
         return self.norm1
 
-    def forward(self, resid, delta, ctx, cache, next_norm=None):
+    def forward(self, resid, delta, ctx, cache, next_norm=None, results=None, position=0):
         if isinstance(delta, Normed):
             if delta.norm is not self.norm1:
                 raise RuntimeError("a finished norm reached another norm than the one it was made for")
@@ -128,12 +155,18 @@ class SandwichBlock(Block):
         else:
             x = self.norm1.add_norm(resid, delta)
         a = self.mixer.forward(x, ctx, cache)
-        if self.feed_forward is None:
-            x = self.norm1b.add_normed(resid, a, next_norm)
-        else:
+        last, out = self.norm1b, a
+        if self.feed_forward is not None:
             x = self.norm1b.add_normed(resid, a, self.norm2)
-            f = self.feed_forward.forward(x, ctx)
-            x = self.norm2b.add_normed(resid, f, next_norm)
+            last, out = self.norm2b, self.feed_forward.forward(x, ctx)
+        if self.depth_average is None:
+            x = last.add_normed(resid, out, next_norm)
+        else:
+            # the same kernel keeps the block's result and leaves the weighted sum of all results in the stream
+            if results is None or position + 2 != self.depth_average.count:
+                raise RuntimeError(f"a depth average of {self.depth_average.count} weights at run-order position "
+                                   f"{position}: it weighs the embedding's rows and one result per block so far")
+            x = last.add_normed(resid, out, next_norm, average=(results, position + 2, self.depth_average.weights))
         return Normed(x, next_norm) if next_norm is not None else None
 
 

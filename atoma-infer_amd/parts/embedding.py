@@ -32,11 +32,11 @@ class TokenEmbedding(Part):
     def device_bytes(self) -> int:
         return 0  # a step reads only the rows of its tokens
 
-    def forward(self, tokens: torch.Tensor, norm=None):
-        """The float32 residual rows of ``tokens``; with ``norm`` (the norm that reads them first) a pair (rows,
-        that norm begun or None)."""
+    def forward(self, tokens: torch.Tensor, norm=None, out=None):
+        """The float32 residual rows of ``tokens`` (into ``out`` where given); with ``norm`` (the norm that reads them
+        first) a pair (rows, that norm begun or None)."""
         if norm is None:
-            return ops.embed(tokens, self.weight)
+            return ops.embed(tokens, self.weight, out)
         got = norm.embed(self.weight, tokens)
         return got if got is not None else (ops.embed(tokens, self.weight), None)
 

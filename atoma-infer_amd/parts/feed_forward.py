@@ -1,4 +1,5 @@
-"""Dense SwiGLU feed-forward: ``down(silu(gate(x)) * up(x))``, no biases (models/src/llama.rs:362-366, 372-374).
+"""Dense gated feed-forward: ``down(act(gate(x)) * up(x))``, no biases; act is SiLU (SwiGLU:
+models/src/llama.rs:362-366, 372-374) or, for designs that ask for it, the tanh form of GELU.
 
 gate and up are fused into one [2 I, width] matrix at load time, so one product feeds the SiLU-multiply kernel.
 When I is a multiple of 16 the rows are interleaved in blocks of 16 (16 gate rows, then the 16 up rows of the
@@ -18,8 +19,12 @@ from .linear import linear, linear_delta
 
 class SwiGLU(FeedForward):
     def __init__(self, width: int, intermediate: int,
-                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight")):
+                 names=("gate_proj.weight", "up_proj.weight", "down_proj.weight"), activation: str = "silu"):
         # ``names``: the tensors of the gate, up and down matrices below the part's prefix
+        # ``activation``: of the gate, "silu" or "gelu_tanh" (0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))))
+        if activation not in ops.GATE_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not supported (known: {', '.join(ops.GATE_ACTIVATIONS)})")
+        self.activation = str(activation)
         self.width, self.inter, self.names = int(width), int(intermediate), tuple(names)
         self.block = 0
         self.w_gate_up: Optional[torch.Tensor] = None
@@ -49,7 +54,8 @@ class SwiGLU(FeedForward):
         self.w_gate_up_tiled = self.w_down_tiled = None
         if act_dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16 and self.w_down.dtype is torch.bfloat16:
             from ..kernels import gemm_bf16
-            plan = gemm_bf16.tiled_plan(2 * self.inter, self.width, swiglu=True) if self.block else None
+            plan = gemm_bf16.tiled_plan(2 * self.inter, self.width, swiglu=True) \
+                if self.block and self.activation == "silu" else None
             if plan is not None:
                 self.w_gate_up_tiled = gemm_bf16.tile_weight(self.w_gate_up, *plan)
             self.w_down_tiled = gemm_bf16.tile_copies_resid(self.w_down)
@@ -62,11 +68,13 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, ctx, sink=None):
         h = None
-        if self.block and x.dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16:
+        # (the products' own epilogue knows SiLU only; another activation runs behind the product)
+        if self.block and x.dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16 \
+                and self.activation == "silu":
             from ..kernels import gemm_bf16
             h = gemm_bf16.try_linear_swiglu(x, self.w_gate_up, self.w_gate_up_tiled)
         if h is None:
-            h = ops.swiglu(linear(x, self.w_gate_up), block=self.block)
+            h = ops.swiglu(linear(x, self.w_gate_up), block=self.block, act=self.activation)
         return linear_delta(h, self.w_down, sink, self.w_down_tiled)
 
 

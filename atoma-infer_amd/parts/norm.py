@@ -14,11 +14,13 @@ from .base import Begun, Norm, WeightedSum, WeightSpec, register_norm
 
 
 class RMSNorm(Norm):
-    def __init__(self, width: int, eps: float, name: str = "weight", offset: float = 0.0):
+    def __init__(self, width: int, eps: float, name: str = "weight", offset: float = 0.0, scalar: bool = False):
         # ``name``: the tensor's name below the part's prefix ("weight" as checkpoints of the Llama family have it)
         # ``offset``: what is added to the stored tensor to make the weight (1 for weights stored around zero); such
         # a weight is kept in float32, since 1 + w has more digits than the checkpoint's dtype
+        # ``scalar``: the checkpoint holds one number for all columns (a tensor without dimensions, or of one entry)
         self.width, self.eps, self.name, self.offset = int(width), float(eps), str(name), float(offset)
+        self.scalar = bool(scalar)
         self.weight: Optional[torch.Tensor] = None
         self.weight_f32: Optional[torch.Tensor] = None
         self.act_dtype = torch.float32
@@ -27,10 +29,12 @@ class RMSNorm(Norm):
         return True
 
     def weight_specs(self) -> Dict[str, WeightSpec]:
-        return {self.name: WeightSpec((self.width,), "norm" if self.offset == 0.0 else "norm_zero")}
+        return {self.name: WeightSpec(() if self.scalar else (self.width,), "norm" if self.offset == 0.0 else "norm_zero")}
 
     def load(self, get, device, act_dtype) -> None:
         self.weight = get(self.name).to(device).contiguous()
+        if self.scalar:      # the kernels take a weight per column: the one number, as often as there are columns
+            self.weight = self.weight.reshape(1).expand(self.width).contiguous()
         if self.offset != 0.0:
             self.weight = (self.weight.to(torch.float32) + self.offset).contiguous()
         self.weight_f32 = self.weight.to(torch.float32)
@@ -49,11 +53,19 @@ class RMSNorm(Norm):
             delta = None
         return ops.add_rmsnorm(resid, delta, self.weight, self.eps, self.act_dtype, rows)
 
-    def add_normed(self, resid, delta, next_norm=None):
+    def add_normed(self, resid, delta, next_norm=None, average=None):
         """``resid += self(delta)`` (in place): this norm stands behind a sublayer, whose output ``delta`` (a tensor,
         float32 planes or a ``WeightedSum`` of up to two such) it norms before the sum.  With ``next_norm`` (an
-        RMSNorm) the same kernel also returns ``next_norm(resid)`` in the activation dtype."""
+        RMSNorm) the same kernel also returns ``next_norm(resid)`` in the activation dtype.  ``average`` = (results
+        float32 [blocks + 1, T, W], n, weights float32 [n]): the new rows are kept as results[n - 1] and the stream
+        becomes ``sum_(j < n) weights[j] results[j]`` before ``next_norm`` reads it."""
         terms = delta.terms if isinstance(delta, WeightedSum) else [(delta, 1.0)]
+        if average is not None:
+            results, n, weights = average
+            if next_norm is None:
+                return ops.depth_average(resid, terms, self.weight_f32, self.eps, results, n, weights)
+            return ops.depth_average(resid, terms, self.weight_f32, self.eps, results, n, weights,
+                                     next_norm.weight_f32, next_norm.eps, next_norm.act_dtype)
         if next_norm is None:
             return ops.add_normed(resid, terms, self.weight_f32, self.eps)
         return ops.add_normed(resid, terms, self.weight_f32, self.eps, next_norm.weight_f32, next_norm.eps,

@@ -214,5 +214,82 @@ class StateSpaceDuality(Mixer):
         return linear_delta(u, self.w_o, sink, self.w_o_tiled)
 
 
+class MinGRU(Mixer):
+    """A gated recurrence whose gates read the current token only (the minGRU form): per channel
+
+        z = sigmoid(W_z h + b_z);   u = W_x h + b_x;   c = u + 1/2 where u >= 0, sigmoid(u) where u < 0;
+        S <- (1 - z) S + z c;       out = W_o (S * silu(W_g h)),
+
+    ``inner`` channels.  A request's state is S, one float32 row, zero at its start.  Gates, candidate and S are
+    float32 in both dtypes; the three input projections are one product in the activation dtype with float32 sums
+    that leaves unrounded.  Since the step is linear in S, entries of many tokens are walked in stretches side by
+    side (``ops.mingru_plan``, made once per step on the host), and decoded tokens by the plain walk.
+
+    Tensors ([out, in]): ``z``, ``x``, ``g`` [inner, width], ``z.b``, ``x.b`` [inner], ``o`` [width, inner].
+    """
+
+    def __init__(self, width: int, inner: int):
+        if inner <= 0:
+            raise ValueError("the recurrence needs at least one channel")
+        self.width, self.inner = int(width), int(inner)
+        self.off_x, self.off_g = self.inner, 2 * self.inner
+        self.w_in = self.w_o = self.w_o_tiled = self.b_z = self.b_x = None
+
+    def graph_safe(self) -> bool:
+        return True     # entries, slots and lengths come from the step's device tensors, stretches from its plan
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        w, n = self.width, self.inner
+        return {"z": WeightSpec((n, w), std=0.08), "z.b": WeightSpec((n,), std=0.5),
+                "x": WeightSpec((n, w), std=0.08), "x.b": WeightSpec((n,), std=0.5),
+                "g": WeightSpec((n, w), std=0.08), "o": WeightSpec((w, n))}
+
+    def state_spec(self) -> StateSpec:
+        return StateSpec((self.inner,), "float32")
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("z"), get("x"), get("g")]
+        dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        parts = [w.to(device=device, dtype=dt) for w in ws]
+        if (-3 * self.inner) % 64:      # whole tiles for the matrix-core products
+            parts.append(torch.zeros(((-3 * self.inner) % 64, self.width), dtype=dt, device=device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        self.b_z, self.b_x = get("z.b").to(**f32).contiguous(), get("x.b").to(**f32).contiguous()
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_o))
+
+    def step_planner(self, page_size: int, cache_dtype: torch.dtype):
+        """(key, fn(starts, counts, bucket_tokens) -> (int32 array, stretches)): the stretches of long entries."""
+        import numpy as np
+        cus = torch.cuda.get_device_properties(self.w_o.device).multi_processor_count
+        blocks = -(-self.inner // 256)
+
+        def plan(starts, counts, bucket):
+            got = ops.mingru_plan(counts, self.inner, cus)
+            return got if got is not None else (np.zeros(0, dtype=np.int32), 0)
+        return ("mingru_stretches", blocks), plan
+
+    def forward(self, x, ctx, cache):
+        proj = linear(x, self.w_in, torch.float32)
+        blocks = -(-self.inner // 256)
+        plan = getattr(ctx, "plans", {}).get(("mingru_stretches", blocks))
+        if plan is None and getattr(ctx, "h_counts", None) is not None:
+            # a caller without a step planner (a kernel test): plan here and now
+            got = ops.mingru_plan(ctx.h_counts, self.inner)
+            if got is not None:
+                plan = (torch.from_numpy(got[0]).to(x.device), got[1])
+        y = ops.mingru(proj, self.off_x, self.off_g, self.inner, self.b_z, self.b_x, ctx.q_start, ctx.state_slots,
+                       cache.state, x.dtype, plan)
+        return linear_delta(y, self.w_o, None, self.w_o_tiled)
+
+
 register_mixer("gated_delta_rule", GatedDeltaRule)
+register_mixer("mingru", MinGRU)
 register_mixer("state_space_duality", StateSpaceDuality)
