@@ -17,7 +17,9 @@ experts) at layer sizes that resemble a real model's, beside the Llama of equal 
 width: prefill of 2,048 tokens and decode steps at batch 1, 8 and 64 through the same engine, ONE line of its own
 (``--sizes 1b|3b`` picks the pair, ``--layers`` how many layers of each, 4 by default; ``--only`` one of the two).
 ``--compare morulix`` does the same for the Morulix decoder (latent attention, a state-space recurrence and windowed
-attention in turn, each beside a dense feed-forward, behind one pass of its loop's entry).
+attention in turn, each beside a dense feed-forward, behind one pass of its loop's entry), and ``--compare rakuvik``
+for the Rakuvik decoder (differential attention and a minGRU recurrence in turn, dense and routed feed-forwards in
+turn, the layers' results averaged over depth).
 
 ``--workload`` runs one of the other two workloads instead and prints ONE line of its own:
 ``serve3b``: Llama-3.2-3B sizes, 64 requests with prompt lengths uniform in [128, 4096] (seeded), 256 generated tokens
@@ -259,6 +261,54 @@ def step_bytes_morulix(model, cfg: dict, batch: int, ctx: float) -> float:
     return total
 
 
+def rakuvik_like(llama: dict, layers: int) -> dict:
+    """The Rakuvik configuration beside ``llama``: the same width and vocabulary; layers in turn differential attention
+    (half as many heads, each of two maps of the Llama's head size over values of twice that, so that queries, keys and
+    values are as wide as the Llama's) before a dense feed-forward of the Llama's width, a minGRU recurrence of twice
+    the model's width before routed experts (squared ReLU, 2,048 columns, as many chosen of eight times as many as
+    make up the dense width, and a shared one), differential attention that reads the first layer's keys and values,
+    and the recurrence again."""
+    w, nh, nkv = llama["hidden_size"], llama["num_attention_heads"], llama["num_key_value_heads"]
+    hd = w // nh
+    ff = 2048
+    top = llama["intermediate_size"] // ff
+    dense = {"kind": "dense", "ff": llama["intermediate_size"]}
+    moe = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": 8 * top, "scale": 2.5, "top": top},
+           "shared": {"ff": ff}}
+    mixer = {"dim": hd, "heads": nh // 2, "kv_heads": max(1, nkv // 2), "vdim": 2 * hd, "scale": hd ** -0.5, "diff": 0.8,
+             "rot": {"base": llama["rope_theta"], "dims": hd, "scaling": {"factor": 4.0}}}
+    out = []
+    for i in range(layers):
+        if i % 2:
+            out.append({"type": "mingru", "mixer": {"width": 2 * w}, "mlp": moe})
+        elif i % 4 == 2:
+            out.append({"type": "attention", "mixer": dict(mixer, kv_from=i - 2), "mlp": dense})
+        else:
+            out.append({"type": "attention", "mixer": mixer, "mlp": dense})
+    return {"architecture": "Rakuvik", "layers": out, "norm": {"eps": 1e-5}, "vocab": llama["vocab_size"], "width": w,
+            "max_positions": llama["max_position_embeddings"]}
+
+
+def step_bytes_rakuvik(model, cfg: dict, batch: int, ctx: float) -> float:
+    """Bytes a decode step of ``batch`` requests at context ``ctx`` has to read (and, for the state, write): every
+    dense matrix once, the experts that ``batch`` tokens are expected to choose between them, the keys of both maps
+    and the values of every attention layer (one that reads another layer's reads them again), the recurrent state
+    twice, and the kept results of all layers once for every layer behind them."""
+    total = float(model.weight_bytes())
+    w = cfg["width"]
+    for i, l in enumerate(cfg["layers"]):
+        m, f = l["mixer"], l["mlp"]
+        if l["type"] == "attention":
+            total += batch * ctx * 2.0 * 2 * m["kv_heads"] * max(2 * m["dim"], m["vdim"])
+        else:
+            total += batch * 2 * 4.0 * m["width"]
+        if f and f["kind"] == "moe":
+            e, top = f["router"]["experts"], f["router"]["top"]
+            total += (e * (1.0 - (1.0 - top / e) ** batch) - top) * 2.0 * 2 * w * f["expert"]["ff"]
+        total += batch * 4.0 * w * (i + 2)
+    return total
+
+
 def compare_main(args) -> int:
     import torch
     import atoma_infer_amd  # noqa: F401
@@ -268,7 +318,7 @@ def compare_main(args) -> int:
     layers = args.layers or 4
     llama = dict(dict(LLAMA_1B, **OTHER_SIZES.get(sizes, {})), num_hidden_layers=layers)
     design = args.compare
-    sun = somesun_like(llama, layers) if design == "somesun" else morulix_like(llama, layers)
+    sun = {"somesun": somesun_like, "morulix": morulix_like, "rakuvik": rakuvik_like}[design](llama, layers)
     out = {}
     for name, cfg in (("llama", llama), (design, sun)):
         if args.only and args.only != name:
@@ -286,6 +336,8 @@ def compare_main(args) -> int:
                 nbytes = step_bytes_somesun(sun, b, ctx)
             elif name == "morulix":
                 nbytes = step_bytes_morulix(model, sun, b, ctx)
+            elif name == "rakuvik":
+                nbytes = step_bytes_rakuvik(model, sun, b, ctx)
             else:
                 nbytes = model.weight_bytes() + kv * ctx * b
             res[f"decode_b{b}_tok_s"] = round(b * st / d, 1)
@@ -295,9 +347,13 @@ def compare_main(args) -> int:
         del model
         torch.cuda.empty_cache()
     l = sun["layers"][0]
-    shown = {"left": l["mixer"]["left"], "right": l["mixer"]["right"], "mlp": l["mlp"]} if design == "somesun" else \
-        {"layers_in_turn": [{"type": x["type"], "mixer": x["mixer"]} for x in sun["layers"][:4]], "mlp": l["mlp"],
-         "loop": sun["loop"]}
+    if design == "somesun":
+        shown = {"left": l["mixer"]["left"], "right": l["mixer"]["right"], "mlp": l["mlp"]}
+    elif design == "morulix":
+        shown = {"layers_in_turn": [{"type": x["type"], "mixer": x["mixer"]} for x in sun["layers"][:4]], "mlp": l["mlp"],
+                 "loop": sun["loop"]}
+    else:
+        shown = {"layers_in_turn": sun["layers"][:4]}
     line = {"metric": f"{design.capitalize()} beside Llama at {sizes} layer sizes, {layers} layers each: prefill of "
                       f"{args.prefill_tokens} tokens, decode at batch 1, 8, 64 ({args.prompt_len}-token prompts)",
             "unit": "tokens/s, ms a step, fraction of 8 TB/s", "n_gpus": 1, "dtype": "bf16",
@@ -364,9 +420,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--workload", choices=["decode", *WORKLOADS], default="decode",
                     help="decode: the default run; serve3b, long8b: the other two workloads, one line of their own")
-    ap.add_argument("--compare", choices=["somesun", "morulix"], default=None,
+    ap.add_argument("--compare", choices=["somesun", "morulix", "rakuvik"], default=None,
                     help="measure that design at --sizes (1b, 3b) beside the Llama of equal sizes, one line of its own")
-    ap.add_argument("--only", choices=["llama", "somesun", "morulix"], default=None, help="with --compare: one of the two models")
+    ap.add_argument("--only", choices=["llama", "somesun", "morulix", "rakuvik"], default=None, help="with --compare: one of the two models")
     ap.add_argument("--requests", type=int, default=0, help="requests of a --workload run (default: the workload's)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the probes of what the GPU delivers")
     ap.add_argument("--chain-floors", action="store_true",
