@@ -45,22 +45,24 @@ diff_prepare_kernel(const TP* __restrict__ proj, int ld, const int32_t* __restri
     cs[i] = c, sn[i] = s;
   }
   __syncthreads();
+  // a token's columns are dealt over the gridDim.y workgroups that share it (steps of few tokens)
+  const int first = blockIdx.y * 256 + threadIdx.x, step = gridDim.y * 256;
   // queries: head j = 2 * head + map, its dim columns at column map * dim of HDO
   const int nq = 2 * heads * hdo;
-  for (int i = threadIdx.x; i < nq; i += 256) {
+  for (int i = first; i < nq; i += step) {
     const int j = i / hdo, c = i - j * hdo;
     const int d = c - (j & 1) * dim;
     float v = 0.f;
     if (d >= 0 && d < dim) v = turned(row + (size_t)j * dim, d, rot_dim, cs, sn);
     q_out[(size_t)t * ldq + i] = from_f32<TQ>(v);
   }
-  for (int h = threadIdx.x; h < heads; h += 256)
+  for (int h = first; h < heads; h += step)
     gate[(size_t)t * heads + h] = 1.0f / (1.0f + expf(-to_f32(row[off_g + h])));
   if (kcache == nullptr) return;
   const int slot = slot_mapping[t];
   const int page = slot / page_size, off = slot % page_size;
   const int nk = kv_heads * hdo;
-  for (int i = threadIdx.x; i < nk; i += 256) {
+  for (int i = first; i < nk; i += step) {
     const int g = i / hdo, c = i - g * hdo;
     const size_t tile = ((size_t)page * kv_heads + g) * page_size * hdo;
     float k = 0.f;
@@ -112,7 +114,11 @@ extern "C" int atoma_diff_prepare(const void* proj, int proj_dtype, int ld, cons
       rot_dim % 2 || rot_dim > dim || rot_dim > 256 || page_size <= 0 || ldq < 2 * heads * hdo || ld < off_g + heads ||
       (kcache != nullptr && (vcache == nullptr || slot_mapping == nullptr)))
     return ATOMA_ERR_SHAPE;
-  dim3 grid(n_tokens), block(256);
+  // steps of few tokens: several workgroups a token, so that about a thousand of them share the step's columns
+  const int per_token = (2 * heads * hdo + 255) / 256;
+  int parts = 1024 / n_tokens;
+  parts = parts < 1 ? 1 : parts > per_token ? per_token : parts > 16 ? 16 : parts;
+  dim3 grid(n_tokens, parts), block(256);
 #define ATOMA_DP(TP, TQ, TC)                                                                                        \
   hipLaunchKernelGGL((diff_prepare_kernel<TP, TQ, TC>), grid, block, 0, stream, (const TP*)proj, ld, positions,     \
                      inv_freq, rot_dim, (TQ*)q_out, ldq, (TC*)kcache, (TC*)vcache, slot_mapping, page_size, gate,   \

@@ -283,6 +283,116 @@ depth_average_kernel(float* __restrict__ resid, Term a, Term b, int n_terms, con
   for (int i = threadIdx.x; i < width; i += 256) out[base + i] = from_f32<TO>(row[i] * inv2 * w_next[i]);
 }
 
+// The same for rows whose width is a multiple of 4 (at most 1024 * MAXJ columns, 16-byte aligned operands): a thread
+// keeps its columns in registers; the earlier results are fetched four at a time, together with the stream's rows
+// and the sublayer's planes, before the first sum over the row, so a step of few rows waits for memory once.
+template <typename TO, int MAXJ>
+__global__ void __launch_bounds__(256)
+depth_average_vec_kernel(float* __restrict__ resid, Term a, Term b, int n_terms, const float* __restrict__ w_post,
+                         const float* __restrict__ earlier, float* __restrict__ kept, size_t result_stride, int n,
+                         const float* __restrict__ dw, const float* __restrict__ w_next, TO* __restrict__ out,
+                         int width, float eps_post, float eps_next) {
+  __shared__ float scratch[4];
+  const size_t base = (size_t)blockIdx.x * width;
+  const int n4 = width >> 2;
+  f4 d[MAXJ], x[MAXJ], acc[MAXJ];
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    d[j] = f4{{0.f, 0.f, 0.f, 0.f}};
+    acc[j] = f4{{0.f, 0.f, 0.f, 0.f}};
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) x[j] = load4(resid + base + 4 * c);
+  }
+  // sum_(j < n - 1) dw[j] * results[j], j ascending
+  for (int s0 = 0; s0 < n - 1; s0 += 4) {
+    f4 r[4][MAXJ];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int s = s0 + q < n - 1 ? s0 + q : n - 2;
+#pragma unroll
+      for (int j = 0; j < MAXJ; ++j) {
+        const int c = threadIdx.x + j * 256;
+        if (c < n4) r[q][j] = load4(earlier + (size_t)s * result_stride + base + 4 * c);
+      }
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (s0 + q < n - 1) {
+        const float w = dw[s0 + q];
+#pragma unroll
+        for (int j = 0; j < MAXJ; ++j)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[j].v[i] += w * r[q][j].v[i];
+      }
+  }
+  if (a.dtype == kF32) add_term<float, MAXJ>(d, a, base, n4);
+  else add_term<bf16_t, MAXJ>(d, a, base, n4);
+  if (n_terms > 1) {
+    if (b.dtype == kF32) add_term<float, MAXJ>(d, b, base, n4);
+    else add_term<bf16_t, MAXJ>(d, b, base, n4);
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j)
+    if (threadIdx.x + j * 256 < n4)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) ss += d[j].v[i] * d[j].v[i];
+  float inv = 1.0f;
+  if (w_post != nullptr) {
+    ss = block_sum<4>(ss, scratch);
+    inv = 1.0f / sqrtf(ss / (float)width + eps_post);
+  }
+  const float last = dw[n - 1];
+  float ss2 = 0.f;
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) {
+      const f4 wp = w_post != nullptr ? load4(w_post + 4 * c) : f4{{1.f, 1.f, 1.f, 1.f}};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) x[j].v[i] += w_post != nullptr ? d[j].v[i] * inv * wp.v[i] : d[j].v[i];
+      store4(kept + base + 4 * c, x[j]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        x[j].v[i] = acc[j].v[i] + last * x[j].v[i];
+        ss2 += x[j].v[i] * x[j].v[i];
+      }
+      store4(resid + base + 4 * c, x[j]);
+    }
+  }
+  if (out == nullptr) return;
+  ss2 = block_sum<4>(ss2, scratch);
+  const float inv2 = 1.0f / sqrtf(ss2 / (float)width + eps_next);
+#pragma unroll
+  for (int j = 0; j < MAXJ; ++j) {
+    const int c = threadIdx.x + j * 256;
+    if (c < n4) {
+      const f4 wn = load4(w_next + 4 * c);
+      f4 y;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y.v[i] = x[j].v[i] * inv2 * wn.v[i];
+      store4(out + base + 4 * c, y);
+    }
+  }
+}
+
+template <typename TO>
+static void launch_depth_vec(dim3 grid, hipStream_t stream, float* resid, const Term& a, const Term& b, int n_terms,
+                             const float* w_post, float* results, size_t result_stride, int n, const float* dw,
+                             const float* w_next, void* out, int width, float eps_post, float eps_next) {
+  const dim3 block(256);
+  float* kept = results + (size_t)(n - 1) * result_stride;
+  if (width <= 2048)
+    hipLaunchKernelGGL((depth_average_vec_kernel<TO, 2>), grid, block, 0, stream, resid, a, b, n_terms, w_post, results,
+                       kept, result_stride, n, dw, w_next, (TO*)out, width, eps_post, eps_next);
+  else if (width <= 4096)
+    hipLaunchKernelGGL((depth_average_vec_kernel<TO, 4>), grid, block, 0, stream, resid, a, b, n_terms, w_post, results,
+                       kept, result_stride, n, dw, w_next, (TO*)out, width, eps_post, eps_next);
+  else
+    hipLaunchKernelGGL((depth_average_vec_kernel<TO, 8>), grid, block, 0, stream, resid, a, b, n_terms, w_post, results,
+                       kept, result_stride, n, dw, w_next, (TO*)out, width, eps_post, eps_next);
+}
+
 extern "C" int atoma_depth_average(float* resid, const void* d0, int dtype0, int planes0, size_t stride0, float scale0,
                                    const void* d1, int dtype1, int planes1, size_t stride1, float scale1,
                                    const float* w_post, float eps_post, float* results, size_t result_stride, int n,
@@ -297,7 +407,17 @@ extern "C" int atoma_depth_average(float* resid, const void* d0, int dtype0, int
   const int n_terms = d1 != nullptr ? 2 : 1;
   const size_t lds = (size_t)width * sizeof(float);
   dim3 grid(n_rows), block(256);
-  if (out == nullptr || out_dtype == kF32)
+  auto aligned = [](const void* p) { return ((uintptr_t)p & 15) == 0; };
+  const bool vec = width % 4 == 0 && width <= 8192 && aligned(resid) && aligned(d0) && aligned(d1) && aligned(w_post) &&
+                   aligned(w_next) && aligned(out) && aligned(results) && result_stride % 4 == 0 && stride0 % 4 == 0 &&
+                   (d1 == nullptr || stride1 % 4 == 0);
+  if (vec && (out == nullptr || out_dtype == kF32))
+    launch_depth_vec<float>(grid, stream, resid, a, b, n_terms, w_post, results, result_stride, n, dw, w_next, out,
+                            width, eps_post, eps_next);
+  else if (vec && out_dtype == kBF16)
+    launch_depth_vec<bf16_t>(grid, stream, resid, a, b, n_terms, w_post, results, result_stride, n, dw, w_next, out,
+                             width, eps_post, eps_next);
+  else if (out == nullptr || out_dtype == kF32)
     hipLaunchKernelGGL((depth_average_kernel<float>), grid, block, lds, stream, resid, a, b, n_terms, w_post, results,
                        result_stride, n, dw, w_next, (float*)out, width, eps_post, eps_next);
   else if (out_dtype == kBF16)
