@@ -90,6 +90,7 @@ struct FuseArgs {
   int gamma_is_bf16;
   uint16_t* u_out;
   float* ss_out;
+  int gate_act;            // the gate's activation in the gate-up epilogue: 0 silu, 1 the tanh form of gelu
 };
 
 // HALF (one tile of W, at most 16 rows of A, the residual epilogue): a wave owns 8 rows of W, not 16, so that twice
@@ -149,6 +150,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
     fa.ss_in = seg->fa.ss_in, fa.parts_in = seg->fa.parts_in, fa.eps_in = seg->fa.eps_in;
     fa.inv_width_in = seg->fa.inv_width_in, fa.resid = seg->fa.resid, fa.gamma = seg->fa.gamma;
     fa.gamma_is_bf16 = seg->fa.gamma_is_bf16, fa.u_out = seg->fa.u_out, fa.ss_out = seg->fa.ss_out;
+    fa.gate_act = seg->fa.gate_act;
 #else
     plane = plane_arg, ra = ra_arg, fa = fa_arg;
 #endif
@@ -406,7 +408,7 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
   if constexpr (SWIGLU) {
     // W holds, for every 16 outputs, 16 gate rows followed by 16 up rows: row tile r is a gate tile, r + 1 its
     // up tile, and the lane that holds gate value (n, row) holds up value (n, row) too.
-    // C[row][n] = silu(gate) * up, with N / 2 columns (the reference: models/src/llama.rs:364).
+    // C[row][n] = act(gate) * up, with N / 2 columns (silu: the reference, models/src/llama.rs:364).
     static_assert(!SWIGLU || (RT % 2 == 0 && sizeof(TC) == 2), "swiglu epilogue needs pairs of tiles, bf16 out");
 #pragma unroll
     for (int r = 0; r < RT; r += 2) {
@@ -419,7 +421,10 @@ gemm_skinny_kernel(const uint16_t* __restrict__ a, const uint16_t* __restrict__ 
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const float g = acc[r][m][i];
-          v[i] = g / (1.0f + expf(-g)) * acc[r + 1][m][i];
+          const float ga = fa.gate_act == 1
+                               ? 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)))
+                               : g / (1.0f + expf(-g));
+          v[i] = ga * acc[r + 1][m][i];
         }
         uint2 o;
         o.x = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
@@ -647,15 +652,17 @@ extern "C" int atoma_gemm_bf16_skinny_tiled_planes(const void* a, const void* w_
 // layout, is the same for every number of rows.
 extern "C" int atoma_gemm_bf16_skinny_swiglu_tiled(const void* a, const void* w_tiled, void* c, int M, int N, int K,
                                                    int lda, int ldc, int rt, int layout_rt, int wk, const float* ss_in,
-                                                   int parts_in, float eps_in, int width_in, hipStream_t stream) {
+                                                   int parts_in, float eps_in, int width_in, int act,
+                                                   hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   static_assert(batch_depth(1, 2, 4) == batch_depth(4, 2, 4) && batch_depth(1, 4, 4) == batch_depth(4, 4, 4) &&
                 batch_depth(2, 2, 4) == batch_depth(3, 4, 4), "one layout for every number of rows");
   if (M > 64 || K <= 0 || wk != 4 || (rt != 2 && rt != 4) || N % (16 * rt) || K % (32 * wk * batch_depth(1, rt, wk)) ||
       (lda & 7) || lda < K || ldc < N / 2 || (ldc & 3) || ((uintptr_t)a & 15) || ((uintptr_t)w_tiled & 15) ||
-      ((uintptr_t)c & 7) || !fuse_in_ok(ss_in, parts_in, eps_in, width_in, M))
+      ((uintptr_t)c & 7) || !fuse_in_ok(ss_in, parts_in, eps_in, width_in, M) || act < 0 || act > 1)
     return ATOMA_ERR_SHAPE;
-  const FuseArgs fa = fuse_in(ss_in, parts_in, eps_in, width_in);
+  FuseArgs fa = fuse_in(ss_in, parts_in, eps_in, width_in);
+  fa.gate_act = act;
   switch ((M + 15) / 16) {
     case 1: return launch_swiglu_tiled<1>(a, w_tiled, c, M, N, K, lda, ldc, rt, layout_rt, fa, stream);
     case 2: return launch_swiglu_tiled<2>(a, w_tiled, c, M, N, K, lda, ldc, rt, layout_rt, fa, stream);
@@ -796,13 +803,14 @@ static int launch_swiglu_mt(const void* a, const void* w, void* c, int M, int N,
 // of 16 (16 gate rows, then the 16 up rows of the same outputs); c is [M, N / 2] bfloat16.  N % 32 == 0.
 extern "C" int atoma_gemm_bf16_skinny_swiglu(const void* a, const void* w, void* c, int M, int N, int K, int lda,
                                              int ldw, int ldc, int rt, int wk, const float* ss_in, int parts_in,
-                                             float eps_in, int width_in, hipStream_t stream) {
+                                             float eps_in, int width_in, int act, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || K <= 0 || K % (32 * wk) || (N & 31) || (lda & 7) || (ldw & 7) || lda < K || ldw < K || ldc < N / 2 ||
       (ldc & 3) || ((uintptr_t)a & 15) || ((uintptr_t)w & 15) || ((uintptr_t)c & 7) ||
-      !fuse_in_ok(ss_in, parts_in, eps_in, width_in, M))
+      !fuse_in_ok(ss_in, parts_in, eps_in, width_in, M) || act < 0 || act > 1)
     return ATOMA_ERR_SHAPE;
-  const FuseArgs fa = fuse_in(ss_in, parts_in, eps_in, width_in);
+  FuseArgs fa = fuse_in(ss_in, parts_in, eps_in, width_in);
+  fa.gate_act = act;
   switch ((M + 15) / 16) {
     case 1: return launch_swiglu_mt<1>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, fa, stream);
     case 2: return launch_swiglu_mt<2>(a, w, c, M, N, K, lda, ldw, ldc, rt, wk, fa, stream);

@@ -357,8 +357,10 @@ def linear_planes(x: torch.Tensor, w: torch.Tensor, tiled: Optional[TiledWeight]
     return out
 
 
-def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor, tiled: Optional[TiledWeight] = None) -> Optional[torch.Tensor]:
-    """silu(gate) * up of x @ w^T in one kernel, for few rows of x; w [2 I, K] is interleaved in blocks of 16.
+def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor, tiled: Optional[TiledWeight] = None,
+                      act: str = "silu") -> Optional[torch.Tensor]:
+    """act(gate) * up of x @ w^T in one kernel, for few rows of x; w [2 I, K] is interleaved in blocks of 16; ``act``
+    is "silu" or "gelu_tanh".
 
     None when the shape is not taken (the caller then runs the product and the activation separately).
     """
@@ -379,6 +381,7 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor, tiled: Optional[TiledWei
         rt = 4
     if (rt, wk) not in ((2, 1), (4, 1), (2, 4), (2, 8), (4, 4)):
         return None
+    code = {"silu": 0, "gelu_tanh": 1}[act]
     out = torch.empty((m, n // 2), dtype=torch.bfloat16, device=x.device)
     if tiled is not None and (tiled.n, tiled.k) == (n, k) and tiled.wk == wk and m <= TILED_SWIGLU_MAX_M:
         # waves of four tiles read a copy made for two as well, and gain on it from 32 rows on (measured over the
@@ -387,11 +390,11 @@ def try_linear_swiglu(x: torch.Tensor, w: torch.Tensor, tiled: Optional[TiledWei
         rt = 4 if tiled.rt == 4 or (m >= TILED_FOUR_TILES_MIN_M and n % 64 == 0) else 2
         _check(lib().atoma_gemm_bf16_skinny_swiglu_tiled(_p(x), _p(tiled.data), _p(out), m, n, k,
                                                          x.stride(0) if m > 1 else k, n // 2, rt, tiled.rt, wk, *begun,
-                                                         _stream()),
+                                                         code, _stream()),
                "gemm_bf16_skinny_swiglu_tiled")
         return out
     _check(lib().atoma_gemm_bf16_skinny_swiglu(_p(x), _p(w), _p(out), m, n, k, x.stride(0) if m > 1 else k,
-                                               w.stride(0), n // 2, rt, wk, *begun, _stream()),
+                                               w.stride(0), n // 2, rt, wk, *begun, code, _stream()),
            "gemm_bf16_skinny_swiglu")
     return out
 

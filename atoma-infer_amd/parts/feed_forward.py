@@ -54,8 +54,7 @@ class SwiGLU(FeedForward):
         self.w_gate_up_tiled = self.w_down_tiled = None
         if act_dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16 and self.w_down.dtype is torch.bfloat16:
             from ..kernels import gemm_bf16
-            plan = gemm_bf16.tiled_plan(2 * self.inter, self.width, swiglu=True) \
-                if self.block and self.activation == "silu" else None
+            plan = gemm_bf16.tiled_plan(2 * self.inter, self.width, swiglu=True) if self.block else None
             if plan is not None:
                 self.w_gate_up_tiled = gemm_bf16.tile_weight(self.w_gate_up, *plan)
             self.w_down_tiled = gemm_bf16.tile_copies_resid(self.w_down)
@@ -68,11 +67,9 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, ctx, sink=None):
         h = None
-        # (the products' own epilogue knows SiLU only; another activation runs behind the product)
-        if self.block and x.dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16 \
-                and self.activation == "silu":
+        if self.block and x.dtype is torch.bfloat16 and self.w_gate_up.dtype is torch.bfloat16:
             from ..kernels import gemm_bf16
-            h = gemm_bf16.try_linear_swiglu(x, self.w_gate_up, self.w_gate_up_tiled)
+            h = gemm_bf16.try_linear_swiglu(x, self.w_gate_up, self.w_gate_up_tiled, self.activation)
         if h is None:
             h = ops.swiglu(linear(x, self.w_gate_up), block=self.block, act=self.activation)
         return linear_delta(h, self.w_down, sink, self.w_down_tiled)
