@@ -364,11 +364,16 @@ def _diff_parts(m, dtype, seed=7, width=64, reader=True, eps=1e-5, boost=None, m
     (attention(dim=20, heads=6, kv_heads=3, vdim=48, scale=0.2, diff=0.3, rot_dims=20, base=30.0, factor=8.0), 4),
     (attention(dim=8, heads=2, kv_heads=1, vdim=40, scale=0.4, diff=0.6, rot_dims=4, base=10.0), 16),
     (attention(dim=64, heads=8, kv_heads=2, vdim=128, scale=0.1, diff=0.35, rot_dims=64, base=1e4, factor=2.0), 16),
+    (attention(dim=40, heads=3, kv_heads=3, vdim=72, scale=0.15, diff=0.25, rot_dims=40, base=300.0, factor=2.5), 16),
+    (attention(dim=48, heads=5, kv_heads=1, vdim=64, scale=0.14, diff=0.7, rot_dims=16, base=1e5), 16),
+    (attention(dim=72, heads=2, kv_heads=2, vdim=160, scale=0.1, diff=0.45, rot_dims=36, base=50.0, factor=16.0), 16),
+    (attention(dim=128, heads=2, kv_heads=1, vdim=200, scale=0.09, diff=0.15, rot_dims=128, base=1e4), 16),
 ])
 def test_differential_attention_alone_and_a_layer_that_reads_its_cache(m, page, dtype):
     """Values narrower than both maps together, as wide, and wider; part of a map rotated, all of it, none; the
-    rotation slowed or not; one head and grouped heads; pages of 4, 16 and 32 tokens; and beside the part that
-    writes the cache one with queries, gates and a difference weight of its own that only reads it."""
+    rotation slowed or not; one head and grouped heads (two to ten query maps a key head); cached heads of 16 to 256
+    columns; pages of 4, 16 and 32 tokens; and beside the part that writes the cache one with queries, gates and a
+    difference weight of its own that only reads it."""
     parts, plains = _diff_parts(m, dtype)
     assert parts[0].cache_spec().head_size == -(-max(2 * m["dim"], m["vdim"]) // 16) * 16
     got, want = _paged_case(parts, plains, dtype, CUTS, page, seed=m["dim"])
