@@ -137,7 +137,7 @@ def test_softmax_scores_chosen_with_the_correction_and_weighed_without(experts, 
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("width, ff", [(64, 48), (40, 20), (128, 96), (200, 1)])
+@pytest.mark.parametrize("width, ff", [(64, 48), (40, 20), (128, 96), (200, 1), (384, 768)])
 def test_gated_feed_forward_with_the_tanh_form_of_gelu(width, ff, dtype):
     from atoma_infer_amd.parts.base import make_part
     part = make_part("feed_forward", "swiglu", width=width, intermediate=ff, names=("gate", "up", "down"),
@@ -157,7 +157,9 @@ def test_gated_feed_forward_with_the_tanh_form_of_gelu(width, ff, dtype):
                                         (40, moe(ff=24, experts=5, top=5, scale=0.5, shared=8)),
                                         (128, moe(ff=64, experts=8, top=3, scale=2.0, shared=0)),
                                         (64, moe(ff=32, experts=1, top=1, scale=1.0, shared=96)),
-                                        (96, moe(ff=40, experts=3, top=1, scale=0.7, shared=20))])
+                                        (96, moe(ff=40, experts=3, top=1, scale=0.7, shared=20)),
+                                        (384, moe(ff=160, experts=32, top=4, scale=1.8, shared=224)),
+                                        (320, moe(ff=96, experts=16, top=3, scale=2.5, shared=64))])
 def test_routed_experts_alone(width, mlp, dtype):
     """Softmax scores, a correction large enough to change the choice, squared-ReLU experts weighed on their outputs,
     no renormalising (all experts chosen: the weights sum to the scale; one expert: its score is 1), and the expert
@@ -177,10 +179,15 @@ def test_routed_experts_alone(width, mlp, dtype):
         got = _flat(part.forward(h.to(DEV, dtype), None))
         if dtype is torch.float32:
             assert _rel(got, want) < PART_TOL[dtype], t
-        else:
-            # (a token whose choice is a close call may go to another expert in bfloat16)
-            e = (got.double() - want).norm(dim=-1) / want.norm(dim=-1).clamp_min(1e-9)
-            assert float(e.median()) < PART_TOL[dtype] and float((e < 2 * PART_TOL[dtype]).double().mean()) >= 0.9, t
+            continue
+        # bfloat16: a token whose choice is a close call may go to another expert; every other token is held to
+        # the tolerance (the router's logits are float32 sums of bfloat16 products: far more exact than the gap asked)
+        e = (got.double() - want).norm(dim=-1) / want.norm(dim=-1).clamp_min(1e-9)
+        choice = torch.softmax(h.double() @ pw["m.router"].T, -1) + pw["m.correction"]
+        ranked = choice.sort(-1, descending=True).values
+        clear = torch.ones(t, dtype=torch.bool) if r["top"] == r["experts"] else \
+            (ranked[:, r["top"] - 1] - ranked[:, r["top"]]) > 2e-3
+        assert float(clear.double().mean()) > 0.8 and float(e[clear].max()) < 2 * PART_TOL[dtype], (t, float(e[clear].max()))
     if 1 < r["top"] < r["experts"]:
         ids, _ = pr.route(h.double(), pw, "m.", r)
         plain_ids = torch.topk(torch.softmax(h.double() @ pw["m.router"].T, -1), r["top"], dim=-1).indices
