@@ -592,3 +592,34 @@ def test_the_trace_program_runs_the_design(dirs, tmp_path):
     a = torch.from_numpy(np.fromfile(os.path.join(out, "0.f32"), dtype="<f4").reshape(2, -1))
     b = torch.from_numpy(np.fromfile(os.path.join(out, "1.f32"), dtype="<f4").reshape(2, -1))
     assert logit_err(a, want[[0, 8]]) < TOL["float32"] and logit_err(b, want[[29, 3]]) < TOL["float32"]
+
+
+def test_the_command_line_writes_random_weights_and_generates(tmp_path):
+    """``random-weights`` from a config.json of the design, then ``generate``: greedy tokens are the plain model's, and
+    sampling with a seed (temperature, top-k, top-p through the framework's sampler) gives the same tokens twice."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, PYTHONPATH=root)
+    cfg_file, d = tmp_path / "config.json", str(tmp_path / "m")
+    cfg_file.write_text(json.dumps(RAK_A))
+    run = lambda *a: subprocess.run([sys.executable, "-m", "atoma_infer_amd", *a], capture_output=True, text=True, env=env,
+                                    timeout=300, cwd=root)
+    proc = run("random-weights", "--config", str(cfg_file), "--out", d, "--seed", "4", "--norm-jitter", "0.1")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    prompt = tokens(9, RAK_A["vocab"], 2)
+    common = ["generate", "--model", d, "--block-size", "16", "--num-gpu-blocks-override", "16", "--max-model-len", "64",
+              "--max-num-batched-tokens", "64", "--max-num-sequences", "4", "--max-new-tokens", "6", "--ignore-eos-token",
+              "--prompt-ids", ",".join(str(t) for t in prompt)]
+    proc = run(*common, "--dtype", "f32", "--greedy")
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = json.loads(proc.stdout.strip().splitlines()[-1])["inference_outputs"][0]["token_ids"]
+    assert got == pr.greedy_generate(prompt, 6, plain_weights(d), plain_config(d))
+    drawn = []
+    for _ in range(2):
+        proc = run(*common, "--dtype", "bf16", "--temperature", "1.5", "--top-k", "20", "--top-p", "0.9", "--random-seed", "11")
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        drawn.append(json.loads(proc.stdout.strip().splitlines()[-1])["inference_outputs"][0]["token_ids"])
+    assert drawn[0] == drawn[1] and len(drawn[0]) == 6 and all(0 <= t < RAK_A["vocab"] for t in drawn[0])
