@@ -623,3 +623,27 @@ def test_the_command_line_writes_random_weights_and_generates(tmp_path):
         assert proc.returncode == 0, proc.stderr[-2000:]
         drawn.append(json.loads(proc.stdout.strip().splitlines()[-1])["inference_outputs"][0]["token_ids"])
     assert drawn[0] == drawn[1] and len(drawn[0]) == 6 and all(0 <= t < RAK_A["vocab"] for t in drawn[0])
+
+
+@pytest.mark.parametrize("kind", ["recurrences only", "attention only", "one recurrence"])
+def test_models_without_a_cache_or_without_a_state(tmp_path, kind):
+    """A model whose layers are all recurrences keeps no pages, one whose layers are all attention no state rows."""
+    att = dict(dim=16, heads=2, kv_heads=1, vdim=24, scale=0.25, diff=0.3, rot_dims=8, base=50.0, factor=2.0)
+    layers = {"recurrences only": [layer("mingru", mingru(48), dense(40)), layer("mingru", mingru(80), None),
+                                   layer("mingru", mingru(24), moe(ff=32, experts=4, top=2, scale=1.2, shared=16))],
+              "attention only": [layer("attention", attention(**att), moe(ff=32, experts=3, top=2, scale=0.9, shared=0)),
+                                 layer("attention", attention(kv_from=0, **att), dense(48)),
+                                 layer("attention", attention(**att), None)],
+              "one recurrence": [layer("mingru", mingru(32), None)]}[kind]
+    d = write_model(str(tmp_path / "m"), config(layers, width=64, vocab=80), 3)
+    reqs = {i: tokens(n, 80, 7 + i) for i, n in enumerate((90, 37, 2))}
+    want = {i: oracle(d, t) for i, t in reqs.items()}
+    sched = [[(0, 70), (1, 2)], [(0, 1), (1, 1), (2, 2)], [(0, 2), (1, 34)], [(0, 17)]]
+    for dtype in ("float32", "bfloat16"):
+        runner = make_runner(d, dtype, 192, 16, 4)
+        got = run_schedule(runner, reqs, sched)
+        e = torch.cat([row_errors(got[i], want[i]) for i in reqs])
+        assert float(e.max()) < TOL[dtype] if dtype == "float32" else \
+            float(e.median()) < TOL[dtype] / 2 and float((e < TOL[dtype]).double().mean()) >= 0.9, (dtype, float(e.max()))
+        runner.manager.check()
+        assert runner.manager.num_requests() == 0
