@@ -8,7 +8,7 @@ a (page, head) tile is contiguous, and the order of its elements is the one in w
 lanes read them (``cache/layout.py`` and csrc/kernels/cache_layout.h state it).
 
 Mixers that declare a ``StateSpec`` get a tensor [slots, *shape] (float32 unless the spec says otherwise) per layer
-call, indexed by the request's state slot.  A ``CacheSpec`` may ask for values of another width than the keys, or for
+call, indexed by the request's state slot; so does an embedding that declares one.  A ``CacheSpec`` may ask for values of another width than the keys, or for
 no second tensor at all.
 """
 from __future__ import annotations
@@ -20,6 +20,10 @@ import torch
 
 from ..parts.base import CacheSpec
 from .manager import CacheManager, GroupGeometry
+
+
+#: the place of the embedding's state among the layer calls' (which count from 0)
+EMBEDDING_CALL = -1
 
 
 @dataclasses.dataclass
@@ -48,6 +52,11 @@ def plan_cache(spec) -> CachePlan:
     index: Dict[CacheSpec, int] = {}
     where: Dict[int, Tuple[int, int, bool]] = {}
     states: Dict[int, Tuple[Tuple[int, ...], str]] = {}
+    # an embedding that keeps something per request (the token before, say) has its state under EMBEDDING_CALL
+    emb_state = getattr(spec.embedding[1], "state_spec", None)
+    st = emb_state() if emb_state is not None else None
+    if st is not None:
+        states[EMBEDDING_CALL] = (tuple(st.shape), st.dtype)
     for pos, call in enumerate(spec.run_order):
         mixer = spec.layers[call.layer][1].mixer
         st = mixer.state_spec()

@@ -653,6 +653,42 @@ extern "C" int atoma_swiglu(const void* gu, void* out, int dtype, int n_tokens, 
 }
 
 // ---------------------------------------------------------------------------------------------
+// The activation of a feed-forward without a gate: out = act(u), act 0: the square of relu.  u may be wider than it
+// is read (row stride ld); the input may be float32 where the output is bfloat16 (a product's unrounded sums).
+template <typename TI, typename TO>
+__global__ void __launch_bounds__(256)
+dense_act_kernel(const TI* __restrict__ u, int ld, TO* __restrict__ out, int inter, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
+    const size_t t = idx / inter;
+    const int i = (int)(idx % inter);
+    const float v = to_f32(u[t * ld + i]);
+    out[idx] = from_f32<TO>(v > 0.f ? v * v : 0.f);
+  }
+}
+
+extern "C" int atoma_dense_act(const void* u, int u_dtype, int ld, void* out, int out_dtype, int n_tokens, int inter,
+                               int act, hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (inter <= 0 || ld < inter || act != 0) return ATOMA_ERR_SHAPE;
+  const size_t total = (size_t)n_tokens * inter;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 65536) blocks = 65536;
+  if (u_dtype == kF32 && out_dtype == kF32)
+    hipLaunchKernelGGL((dense_act_kernel<float, float>), dim3(blocks), dim3(256), 0, stream, (const float*)u, ld,
+                       (float*)out, inter, total);
+  else if (u_dtype == kF32 && out_dtype == kBF16)
+    hipLaunchKernelGGL((dense_act_kernel<float, bf16_t>), dim3(blocks), dim3(256), 0, stream, (const float*)u, ld,
+                       (bf16_t*)out, inter, total);
+  else if (u_dtype == kBF16 && out_dtype == kBF16)
+    hipLaunchKernelGGL((dense_act_kernel<bf16_t, bf16_t>), dim3(blocks), dim3(256), 0, stream, (const bf16_t*)u, ld,
+                       (bf16_t*)out, inter, total);
+  else
+    return ATOMA_ERR_DTYPE;
+  ATOMA_LAUNCH_CHECK();
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------
 // dst[dst_idx[i]] = src[src_idx[i]]: puts tokens sampled by the previous step, which the host has not seen yet,
 // into the next step's token list on the device.  pairs = [n][2] (dst index, src index).
 __global__ void feed_tokens_kernel(int32_t* __restrict__ dst, const int32_t* __restrict__ src,

@@ -10,7 +10,8 @@
 //                    differ in the order of their elements only), the heads' gates sigmoid(g) in float32, and q in
 //                    the activation dtype;
 //   head_linear      per head a product of its own: out[t, h, :] = W[h] x[t, h, :], optionally times a scalar per
-//                    (token, head), float32 sums in an order that depends on the sizes alone.
+//                    (token, head) or per (token, output column), float32 sums in an order that depends on the sizes
+//                    alone.
 #include "common.h"
 #include "cache_layout.h"
 
@@ -51,7 +52,7 @@ latent_prepare_kernel(const float* __restrict__ proj, int ldp, int off_q, int of
 template <typename TA, typename TW, typename TO>
 __global__ void __launch_bounds__(256)
 head_linear_kernel(const TA* __restrict__ x, int ldx, const TW* __restrict__ w, TO* __restrict__ out, int ldo,
-                   const float* __restrict__ gate, int T, int H, int K, int N) {
+                   const float* __restrict__ gate, int gate_cols, int T, int H, int K, int N) {
   __shared__ float xs[16][33], ws[64][33];
   const int h = blockIdx.z, n0 = blockIdx.x * 64, t0 = blockIdx.y * 16;
   const int nl = threadIdx.x & 63, rg = threadIdx.x >> 6;
@@ -79,7 +80,7 @@ head_linear_kernel(const TA* __restrict__ x, int ldx, const TW* __restrict__ w, 
   for (int i = 0; i < 4; ++i) {
     const int t = t0 + rg + 4 * i;
     if (t < T) {
-      const float s = gate ? gate[(size_t)t * H + h] : 1.0f;
+      const float s = !gate ? 1.0f : gate_cols ? gate[((size_t)t * H + h) * N + n0 + nl] : gate[(size_t)t * H + h];
       out[(size_t)t * ldo + (size_t)h * N + n0 + nl] = from_f32<TO>(acc[i] * s);
     }
   }
@@ -97,7 +98,7 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 template <typename TO, int NS>
 __global__ void __launch_bounds__(256)
 head_linear_mfma_kernel(const uint16_t* __restrict__ x, int ldx, const uint16_t* __restrict__ w, TO* __restrict__ out,
-                        int ldo, const float* __restrict__ gate, int T, int H, int K, int N) {
+                        int ldo, const float* __restrict__ gate, int gate_cols, int T, int H, int K, int N) {
   const int h = blockIdx.z, n0 = blockIdx.x * (16 * NS);
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r16 = lane & 15, kg = lane >> 4;
@@ -137,14 +138,15 @@ head_linear_mfma_kernel(const uint16_t* __restrict__ x, int ldx, const uint16_t*
   }
   t = tb + r16;
   if (t >= T) return;
-  const float g = gate ? gate[(size_t)t * H + h] : 1.0f;
+  const float g = gate && !gate_cols ? gate[(size_t)t * H + h] : 1.0f;
 #pragma unroll
   for (int s = 0; s < NS; ++s) {
     const int nb = n0 + s * 16 + kg * 4;
     TO* dst = out + (size_t)t * ldo + (size_t)h * N + nb;
+    const float* gc = gate + ((size_t)t * H + h) * N + nb;      // (read only with a gate per column)
 #pragma unroll
     for (int i = 0; i < 4; ++i)
-      if (nb + i < N) dst[i] = from_f32<TO>(acc[s][i] * g);
+      if (nb + i < N) dst[i] = from_f32<TO>(acc[s][i] * (gate && gate_cols ? gc[i] : g));
   }
 }
 
@@ -168,7 +170,7 @@ extern "C" int atoma_latent_prepare(const float* proj, int ldp, int off_q, int o
 }
 
 extern "C" int atoma_head_linear(const void* x, int x_dtype, int ldx, const void* w, int w_dtype, void* out,
-                                 int out_dtype, int ldo, const float* gate, int T, int H, int K, int N,
+                                 int out_dtype, int ldo, const float* gate, int gate_cols, int T, int H, int K, int N,
                                  hipStream_t stream) {
   if (T <= 0) return 0;
   if (H <= 0 || K <= 0 || N <= 0 || ldx < H * K || ldo < H * N || H > 65535 || (T + 15) / 16 > 65535) return ATOMA_ERR_SHAPE;
@@ -178,7 +180,7 @@ extern "C" int atoma_head_linear(const void* x, int x_dtype, int ldx, const void
     dim3 mgrid((N + (wide ? 127 : 63)) / (wide ? 128 : 64), (T + 63) / 64, H);
 #define ATOMA_HLM(TO, NS)                                                                                          \
   hipLaunchKernelGGL((head_linear_mfma_kernel<TO, NS>), mgrid, dim3(256), 0, stream, (const uint16_t*)x, ldx,      \
-                     (const uint16_t*)w, (TO*)out, ldo, gate, T, H, K, N)
+                     (const uint16_t*)w, (TO*)out, ldo, gate, gate_cols, T, H, K, N)
     if (out_dtype == kBF16) {
       if (wide) ATOMA_HLM(bf16_t, 8);
       else ATOMA_HLM(bf16_t, 4);
@@ -195,7 +197,7 @@ extern "C" int atoma_head_linear(const void* x, int x_dtype, int ldx, const void
   dim3 grid((N + 63) / 64, (T + 15) / 16, H), block(256);
 #define ATOMA_HL(TA, TW, TO)                                                                                  \
   hipLaunchKernelGGL((head_linear_kernel<TA, TW, TO>), grid, block, 0, stream, (const TA*)x, ldx, (const TW*)w, \
-                     (TO*)out, ldo, gate, T, H, K, N)
+                     (TO*)out, ldo, gate, gate_cols, T, H, K, N)
   if (x_dtype == kF32 && w_dtype == kF32 && out_dtype == kF32) ATOMA_HL(float, float, float);
   else if (x_dtype == kF32 && w_dtype == kBF16 && out_dtype == kF32) ATOMA_HL(float, bf16_t, float);
   else if (x_dtype == kBF16 && w_dtype == kBF16 && out_dtype == kBF16) ATOMA_HL(bf16_t, bf16_t, bf16_t);

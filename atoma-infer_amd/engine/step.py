@@ -197,10 +197,16 @@ class ModelRunner:
         # planners of the mixers, one per distinct key
         self._planners: Dict[object, Callable] = {}
         for _, block in model.spec.layers:
+            # (a mixer of several branches may plan for each: ``step_planners`` gives them all)
+            many = getattr(block.mixer, "step_planners", None)
             plan = getattr(block.mixer, "step_planner", None)
-            got = plan(pool.page_size, pool.dtype) if plan is not None else None
-            if got is not None:
-                self._planners.setdefault(got[0], got[1])
+            if many is not None:
+                found = many(pool.page_size, pool.dtype)
+            else:
+                got = plan(pool.page_size, pool.dtype) if plan is not None else None
+                found = [got] if got is not None else []
+            for key, fn in found:
+                self._planners.setdefault(key, fn)
 
     # -- requests ------------------------------------------------------------------------------------
     def add_request(self, request: int) -> int:

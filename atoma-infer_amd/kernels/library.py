@@ -56,6 +56,10 @@ HIP_MODULES: Dict[str, Tuple[Sequence[str], Sequence[str]]] = {
     "latent": (("latent.hip",), ()),
     "differential": (("differential.hip",), ()),
     "mingru": (("mingru.hip",), ()),
+    "streams": (("streams.hip",), ()),
+    "gated_attention": (("gated_attention.hip",), ()),
+    "lightning": (("lightning.hip",), ()),
+    "rglru": (("rglru.hip",), ()),
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}

@@ -635,18 +635,21 @@ def latent_prepare(proj: torch.Tensor, offsets, heads: int, dim: int, rank: int,
 def head_linear(x: torch.Tensor, w: torch.Tensor, out_dtype: torch.dtype, gate: Optional[torch.Tensor] = None,
                 ) -> torch.Tensor:
     """Per head a product of its own: x [T, H K] (row stride free), w [H, N, K] -> [T, H N] in ``out_dtype``, float32
-    sums; with ``gate`` float32 [T, H] every head's result is multiplied by its number."""
+    sums; with ``gate`` float32 [T, H] every head's result is multiplied by its number, with ``gate`` [T, H N] every
+    output by its own."""
     _dev(x, w, gate)
     _need(w.dim() == 3 and w.is_contiguous(), "head_linear: w must be contiguous [H, N, K]")
     h, n, k = w.shape
     t = x.shape[0]
     _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[1] == h * k, "head_linear: x must be [T, H K]")
+    gate_cols = 0
     if gate is not None:
-        _f32(gate, "gate", t * h)
+        gate_cols = int(gate.numel() == t * h * n and n > 1)
+        _f32(gate, "gate", t * h * n if gate_cols else t * h)
     out = torch.empty((t, h * n), dtype=out_dtype, device=x.device)
     _check(_module("latent").atoma_head_linear(_p(x), _code(x, "x"), x.stride(0) if t > 1 else h * k, _p(w), _code(w, "w"),
-                                               _p(out), _code(out, "out"), h * n, _p(gate), t, h, k, n, _stream()),
-           "head_linear")
+                                               _p(out), _code(out, "out"), h * n, _p(gate), gate_cols, t, h, k, n,
+                                               _stream()), "head_linear")
     return out
 
 
@@ -905,6 +908,311 @@ def mingru(proj: torch.Tensor, off_x: int, off_g: int, width: int, bz: torch.Ten
                                       _p(state), _p(ab), _p(y), _code(y, "y"), width, n_entries, width, int(off_x),
                                       int(off_g), _stream()), "mingru_stretched")
     return y
+
+
+# -- a stream kept in several copies, and the embedding that starts it ------------------------------------------
+
+MAX_STREAM_COPIES = 8
+
+
+def _planes(y: torch.Tensor, t: int, width: int, what: str):
+    _need(y.is_contiguous() and y.dim() in (2, 3) and tuple(y.shape[-2:]) == (t, width),
+          f"{what} must be contiguous [T, W] or [planes, T, W]")
+    return y.shape[0] if y.dim() == 3 else 1
+
+
+def stream_step(x: torch.Tensor, update=None, read=None, rows: Optional[torch.Tensor] = None,
+                out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
+    """One pass over the copies x float32 [S, T, W] of the residual stream.
+
+    ``update`` = (y, mix float32 [S, S] indexed [from, to], out float32 [S]): every copy becomes
+    ``sum_s mix[s, t] x_s + out[t] y``, all from the old ones; y is [T, W] or float32 planes [P, T, W] (summed).
+    ``read`` = (w_in float32 [S], norm weight float32 [W], eps): returns ``rmsnorm(sum_s w_in[s] x_s) * weight`` of the
+    new copies in ``out_dtype``.  With ``rows`` (int32) only those rows are read and x is left as it was."""
+    _need(x.dtype is torch.float32 and x.dim() == 3 and x.is_contiguous(), "the stream must be float32 [S, T, W]")
+    s, t, width = x.shape
+    _need(1 <= s <= MAX_STREAM_COPIES, f"1 to {MAX_STREAM_COPIES} copies of the stream")
+    _need(update is not None or read is not None, "stream_step: nothing to do")
+    y = mix = outw = inw = nw = h = None
+    planes, eps = 0, 0.0
+    if update is not None:
+        y, mix, outw = update
+        planes = _planes(y, t, width, "the sublayer's output")
+        _f32(mix, "mix", s * s)
+        _f32(outw, "out weights", s)
+    if read is not None:
+        inw, nw, eps = read
+        _f32(inw, "in weights", s)
+        _f32(nw, "norm weight", width)
+        n = rows.numel() if rows is not None else t
+        h = torch.empty((n, width), dtype=out_dtype, device=x.device)
+    if rows is not None:
+        _i32(rows, "rows")
+        _need(read is not None, "rows are for reading")
+    _dev(x, y, mix, outw, inw, nw, rows)
+    _check(_module("streams").atoma_stream_step(
+        _p(x), t, width, s, _p(y), _code(y, "y") if y is not None else F32, planes, ctypes.c_size_t(t * width),
+        _p(mix), _p(outw), _p(inw), _p(nw), ctypes.c_float(eps), _p(h), _code(h, "out") if h is not None else F32,
+        _p(rows), rows.numel() if rows is not None else 0, int(rows is None), _stream()), "stream_step")
+    return h
+
+
+def bigram_embed(tokens, positions, token_seq, q_start, state_slots, state: Optional[torch.Tensor],
+                 table: torch.Tensor, pairs: Optional[torch.Tensor], buckets: int, mul_prev: int, mul_cur: int,
+                 scale: float, copies: int) -> torch.Tensor:
+    """x float32 [copies, T, W], every copy ``table[token] * scale + pairs[(prev * mul_prev + token * mul_cur) mod
+    buckets]`` (row ``buckets`` of ``pairs`` at position 0; ``pairs`` None: the first term alone).  ``state`` int32
+    [slots, 1] holds each request's last token between steps."""
+    _dev(tokens, positions, token_seq, q_start, state_slots, state, table, pairs)
+    t, s = tokens.numel(), state_slots.numel()
+    _i32(tokens, "tokens")
+    _i32(positions, "positions", t)
+    _i32(token_seq, "token_seq", t)
+    _i32(q_start, "q_start", s + 1)
+    _i32(state_slots, "state_slots")
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be contiguous [vocab, width]")
+    width = table.shape[1]
+    if pairs is not None:
+        _need(pairs.is_contiguous() and tuple(pairs.shape) == (buckets + 1, width) and pairs.dtype is table.dtype,
+              "the pair table must be [buckets + 1, width] of the embedding's dtype")
+        _need(state is not None and state.dtype is torch.int32 and state.is_contiguous() and state.dim() == 2
+              and state.shape[1] == 1, "the previous-token state must be int32 [slots, 1]")
+    x = torch.empty((copies, t, width), dtype=torch.float32, device=table.device)
+    _check(_module("streams").atoma_bigram_embed(
+        _p(tokens), _p(positions), _p(token_seq), _p(q_start), _p(state_slots), _p(state), _p(table),
+        _code(table, "embedding table"), table.shape[0], _p(pairs), int(buckets), ctypes.c_longlong(mul_prev),
+        ctypes.c_longlong(mul_cur), ctypes.c_float(scale), _p(x), t, int(copies), width, _stream()), "bigram_embed")
+    return x
+
+
+def normed_branches(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, eps: float, scale: float,
+                    bias_a: Optional[torch.Tensor] = None, bias_b: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """float32 [T, W]: ``scale * (rmsnorm(a + bias_a) * wa + rmsnorm(b + bias_b) * wb)``; a and b are [T, W] or
+    float32 planes [P, T, W] (summed first)."""
+    t, width = a.shape[-2:]
+    pa, pb = _planes(a, t, width, "a branch"), _planes(b, t, width, "a branch")
+    _dev(a, b, wa, wb, bias_a, bias_b)
+    _f32(wa, "norm weight", width)
+    _f32(wb, "norm weight", width)
+    for bias in (bias_a, bias_b):
+        if bias is not None:
+            _f32(bias, "bias", width)
+    y = torch.empty((t, width), dtype=torch.float32, device=a.device)
+    _check(_module("streams").atoma_normed_branches(_p(a), _code(a, "a"), pa, _p(b), _code(b, "b"), pb, _p(bias_a),
+                                                    _p(bias_b), _p(wa), _p(wb), ctypes.c_float(eps),
+                                                    ctypes.c_float(scale), _p(y), t, width, _stream()),
+           "normed_branches")
+    return y
+
+
+def dense_act(u: torch.Tensor, out_dtype: torch.dtype, act: str = "relu2") -> torch.Tensor:
+    """act(u) for u [T, I] (float32 or bfloat16) in ``out_dtype``; ``act``: "relu2", the square of relu."""
+    _dev(u)
+    _need(act == "relu2", f"dense_act: unknown activation {act!r}")
+    _need(u.dim() == 2 and u.stride(1) == 1, "dense_act: u must be [T, I]")
+    t, inter = u.shape
+    out = torch.empty((t, inter), dtype=out_dtype, device=u.device)
+    _check(core().atoma_dense_act(_p(u), _code(u, "u"), u.stride(0) if t > 1 else inter, _p(out), _code(out, "out"), t,
+                                  inter, 0, _stream()), "dense_act")
+    return out
+
+
+# -- gated attention kinds: the kernels between projections and attention ---------------------------------------
+
+def _tiles_ok(kcache, vcache, nkv, page_size, hd):
+    pages = kcache.shape[0]
+    _need(kcache.is_contiguous() and vcache is not None and vcache.is_contiguous()
+          and tuple(kcache.shape) == (pages, nkv, page_size * hd) and tuple(vcache.shape) == tuple(kcache.shape)
+          and kcache.dtype is vcache.dtype, "cache tensors must be [pages, kv_heads, page_size * head] tiles of one dtype")
+
+
+def tied_rope_prepare(proj: torch.Tensor, offsets, bq, bk, positions, freq: torch.Tensor, rot: int, interleaved: bool,
+                      mag: float, kcache, vcache, slot_mapping, page_size: int, nh: int, nkv: int, hd: int,
+                      hd_out: int, act_dtype: torch.dtype):
+    """(q [T, nh hd_out] in ``act_dtype``, gate float32 [T, nh hd] = sigmoid) from ``proj`` float32 [T, ld] whose
+    columns ``offsets`` = (q, k, g) name; k with its bias goes into the value tiles as it is and rotated into the key
+    tiles (see gated_attention.hip)."""
+    _dev(proj, bq, bk, positions, freq, kcache, vcache, slot_mapping)
+    t = proj.shape[0]
+    off_q, off_k, off_g = (int(o) for o in offsets)
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "proj must be float32 [T, ld]")
+    _need(min(off_q, off_k, off_g) >= 0 and max(off_q + nh * hd, off_k + nkv * hd, off_g + nh * hd) <= proj.shape[1],
+          "the projections' columns do not fit proj")
+    if bq is not None:
+        _f32(bq, "q bias", nh * hd)
+    if bk is not None:
+        _f32(bk, "k bias", nkv * hd)
+    _i32(positions, "positions", t)
+    _i32(slot_mapping, "slot_mapping", t)
+    _f32(freq, "frequencies", rot // 2)
+    _tiles_ok(kcache, vcache, nkv, page_size, hd_out)
+    _need(kcache.dtype is act_dtype, "the cache must be of the activation dtype")
+    q = torch.empty((t, nh * hd_out), dtype=act_dtype, device=proj.device)
+    gate = torch.empty((t, nh * hd), dtype=torch.float32, device=proj.device)
+    _check(_module("gated_attention").atoma_tied_rope_prepare(
+        _p(proj), proj.stride(0), off_q, off_k, off_g, _p(bq), _p(bk), _p(positions), _p(freq), int(rot),
+        int(bool(interleaved)), ctypes.c_float(mag), _p(q), _code(q, "q"), _p(kcache), _p(vcache),
+        _code(kcache, "cache"), _p(slot_mapping), int(page_size), _p(gate), t, nh, nkv, hd, hd_out, _stream()),
+        "tied_rope_prepare")
+    return q, gate
+
+
+def latent_rope_prepare(proj: torch.Tensor, offsets, q_rank: int, rank: int, rd: int, rank_p: int, n_gate: int,
+                        wq: torch.Tensor, wc: torch.Tensor, eps: float, positions, freq: torch.Tensor, rot: int,
+                        kcache, vcache, slot_mapping, page_size: int, act_dtype: torch.dtype):
+    """(cq [T, q_rank] in ``act_dtype``, gate float32 [T, n_gate] = sigmoid) from ``proj`` float32 [T, ld] whose columns
+    ``offsets`` = (query latent, key/value latent followed by the rotated key part, gates) name; the cache tiles
+    receive [c | rotated part | 0] as the key and [c | 0] as the value, ``rank_p`` columns each."""
+    _dev(proj, wq, wc, positions, freq, kcache, vcache, slot_mapping)
+    t = proj.shape[0]
+    off_dq, off_c, off_g = (int(o) for o in offsets)
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "proj must be float32 [T, ld]")
+    _need(min(off_dq, off_c, off_g) >= 0 and max(off_dq + q_rank, off_c + rank + rd, off_g + n_gate) <= proj.shape[1],
+          "the projections' columns do not fit proj")
+    _f32(wq, "norm weight", q_rank)
+    _f32(wc, "norm weight", rank)
+    _i32(positions, "positions", t)
+    _i32(slot_mapping, "slot_mapping", t)
+    _f32(freq, "frequencies", rot // 2)
+    _tiles_ok(kcache, vcache, 1, page_size, rank_p)
+    _need(kcache.dtype is act_dtype, "the cache must be of the activation dtype")
+    cq = torch.empty((t, q_rank), dtype=act_dtype, device=proj.device)
+    gate = torch.empty((t, n_gate), dtype=torch.float32, device=proj.device)
+    _check(_module("gated_attention").atoma_latent_rope_prepare(
+        _p(proj), proj.stride(0), off_dq, off_c, off_g, q_rank, rank, rd, rank_p, n_gate, _p(wq), _p(wc),
+        ctypes.c_float(eps), _p(positions), _p(freq), int(rot), _p(cq), _code(cq, "cq"), _p(kcache), _p(vcache),
+        _code(kcache, "cache"), _p(slot_mapping), int(page_size), _p(gate), t, _stream()), "latent_rope_prepare")
+    return cq, gate
+
+
+def latent_q_rope(q: torch.Tensor, positions, freq: torch.Tensor, rot: int, heads: int, dim: int, rd: int,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """q float32 [T, heads (dim + rd)] in ``out_dtype`` with the first ``rot`` of every head's last ``rd`` columns
+    rotated in neighbouring pairs."""
+    _dev(q, positions, freq)
+    t = q.shape[0]
+    _need(q.dtype is torch.float32 and q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= heads * (dim + rd),
+          "q must be float32 [T, heads (dim + rd)]")
+    _i32(positions, "positions", t)
+    _f32(freq, "frequencies", rot // 2)
+    out = torch.empty((t, heads * (dim + rd)), dtype=out_dtype, device=q.device)
+    _check(_module("gated_attention").atoma_latent_q_rope(_p(q), q.stride(0), _p(positions), _p(freq), int(rot), _p(out),
+                                                          _code(out, "out"), t, heads, dim, rd, _stream()),
+           "latent_q_rope")
+    return out
+
+
+def gate_mul(att: torch.Tensor, gate: torch.Tensor, heads: int, vd: int, hd_out: int) -> torch.Tensor:
+    """[T, heads vd]: the first ``vd`` of every head's ``hd_out`` columns of ``att`` times ``gate`` float32 [T, heads vd]."""
+    _dev(att, gate)
+    t = att.shape[0]
+    _need(att.is_contiguous() and tuple(att.shape) == (t, heads * hd_out), "att must be contiguous [T, heads hd_out]")
+    _f32(gate, "gate", t * heads * vd)
+    y = torch.empty((t, heads * vd), dtype=att.dtype, device=att.device)
+    _check(_module("gated_attention").atoma_gate_mul(_p(att), _p(gate), _p(y), _code(att, "att"), t, heads, vd, hd_out,
+                                                     _stream()), "gate_mul")
+    return y
+
+
+# -- recurrences with a decay per head or per channel -----------------------------------------------------------
+
+def lightning_scan(proj: torch.Tensor, offsets, q_start, state_slots, state: torch.Tensor, decay: torch.Tensor,
+                   heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """o float32 [T, heads vdim] of the recurrence S <- decay_h S + k v^T, o = S^T q over a step's entries; q, k, v are
+    the SiLU of ``proj``'s columns at ``offsets`` = (q, k, v); each request's S is its row of ``state`` float32
+    [slots, heads * vdim * dim]."""
+    _dev(proj, q_start, state_slots, state, decay)
+    t = proj.shape[0]
+    n_entries = state_slots.numel()
+    off_q, off_k, off_v = (int(o) for o in offsets)
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1, "proj must be float32 [T, ld]")
+    _need(min(off_q, off_k, off_v) >= 0 and max(off_q + heads * dim, off_k + heads * dim, off_v + heads * vdim)
+          <= proj.shape[1], "the projections' columns do not fit proj")
+    _need(dim <= 256, "lightning_scan: key sizes beyond 256 are not supported")
+    _i32(q_start, "q_start", n_entries + 1)
+    _i32(state_slots, "state_slots")
+    _f32(decay, "decay", heads)
+    _need(state.dtype is torch.float32 and state.is_contiguous() and state.dim() == 2
+          and state.shape[1] == heads * vdim * dim, "the state must be float32 [slots, heads * vdim * dim]")
+    o = torch.empty((t, heads * vdim), dtype=torch.float32, device=proj.device)
+    _check(_module("lightning").atoma_lightning_scan(_p(proj), proj.stride(0) if t > 1 else proj.shape[1], off_q, off_k,
+                                                     off_v, _p(q_start), _p(state_slots), _p(state), _p(decay), _p(o),
+                                                     n_entries, heads, dim, vdim, _stream()), "lightning_scan")
+    return o
+
+
+def lightning_out(o: torch.Tensor, proj: torch.Tensor, off_g: int, w: torch.Tensor, eps: float,
+                  out_dtype: torch.dtype) -> torch.Tensor:
+    """rmsnorm(o) * w * sigmoid(proj[:, off_g:]) in ``out_dtype``, the norm over all of a token's columns."""
+    _dev(o, proj, w)
+    t, n = o.shape
+    _f32(o, "o")
+    _f32(w, "norm weight", n)
+    _need(proj.dtype is torch.float32 and proj.stride(1) == 1 and proj.shape[1] >= off_g + n, "the gates do not fit proj")
+    y = torch.empty((t, n), dtype=out_dtype, device=o.device)
+    _check(_module("lightning").atoma_lightning_out(_p(o), _p(proj), proj.stride(0) if t > 1 else proj.shape[1],
+                                                    int(off_g), _p(w), ctypes.c_float(eps), _p(y), _code(y, "y"), t, n,
+                                                    _stream()), "lightning_out")
+    return y
+
+
+def rglru_conv(proj: torch.Tensor, off_y: int, off_x: int, by, bx, conv, conv_b, token_seq, q_start, state_slots,
+               state: torch.Tensor, width: int, taps: int):
+    """(u, g) float32 [T, width]: the convolution of the x branch (its inputs before an entry from the request's row
+    of ``state`` float32 [slots, taps * width], which also takes the inputs for the next step) and gelu of the y
+    branch (see rglru.hip)."""
+    _dev(proj, by, bx, conv, conv_b, token_seq, q_start, state_slots, state)
+    t = proj.shape[0]
+    n_entries = state_slots.numel()
+    _need(proj.dtype is torch.float32 and proj.dim() == 2 and proj.stride(1) == 1
+          and proj.shape[1] >= max(off_y, off_x) + width, "rglru: bad projection")
+    for b, what in ((by, "y bias"), (bx, "x bias"), (conv_b, "convolution bias")):
+        _f32(b, what, width)
+    _f32(conv, "convolution", width * taps)
+    _i32(token_seq, "token_seq", t)
+    _i32(q_start, "q_start", n_entries + 1)
+    _i32(state_slots, "state_slots")
+    _need(state.dtype is torch.float32 and state.is_contiguous() and state.dim() == 2
+          and state.shape[1] == taps * width, "the state must be float32 [slots, taps * width]")
+    u = torch.empty((t, width), dtype=torch.float32, device=proj.device)
+    g = torch.empty((t, width), dtype=torch.float32, device=proj.device)
+    _check(_module("rglru").atoma_rglru_conv(_p(proj), proj.stride(0) if t > 1 else proj.shape[1], int(off_y), int(off_x),
+                                             _p(by), _p(bx), _p(conv), _p(conv_b), _p(token_seq), _p(q_start),
+                                             _p(state_slots), _p(state), _p(u), _p(g), t, n_entries, width, taps,
+                                             _stream()), "rglru_conv")
+    return u, g
+
+
+def rglru_scan(gates: torch.Tensor, u: torch.Tensor, g: torch.Tensor, ba, bi, sp, q_start, state_slots,
+               state: torch.Tensor, blocks: int, taps: int, out_dtype: torch.dtype, plan=None) -> torch.Tensor:
+    """[T, width] = S * g with S <- a S + sqrt(1 - a^2) i u, a = exp(-8 r sp), r and i the sigmoids of ``gates``
+    float32 [T, 2 width] (per block [r | i]) plus ``ba``, ``bi``.  ``plan``: (int32 device tensor, stretches) from
+    ``mingru_plan`` for steps with long entries, or None for the plain walk."""
+    _dev(gates, u, g, ba, bi, sp, q_start, state_slots, state)
+    t, width = u.shape
+    n_entries = state_slots.numel()
+    _f32(gates, "gates", t * 2 * width)
+    _f32(u, "u")
+    _f32(g, "g", t * width)
+    for b, what in ((ba, "gate bias"), (bi, "gate bias"), (sp, "softplus(lam)")):
+        _f32(b, what, width)
+    _i32(q_start, "q_start", n_entries + 1)
+    _i32(state_slots, "state_slots")
+    _need(state.dtype is torch.float32 and state.is_contiguous() and state.dim() == 2
+          and state.shape[1] == taps * width and width % blocks == 0, "the state must be float32 [slots, taps * width]")
+    out = torch.empty((t, width), dtype=out_dtype, device=u.device)
+    arr, n_st, first, ab = None, 0, None, None
+    if plan is not None and plan[1] > 0:
+        arr, n_st = plan
+        _i32(arr, "stretches", 3 * n_st + n_entries + 1)
+        first = ctypes.c_void_p(arr.data_ptr() + 12 * n_st)
+        ab = torch.empty((n_st, 2, width), dtype=torch.float32, device=u.device)
+    _check(_module("rglru").atoma_rglru_scan(_p(gates), 2 * width, _p(u), _p(g), _p(ba), _p(bi), _p(sp), _p(q_start),
+                                             _p(state_slots), _p(state), _p(arr), int(n_st),
+                                             first if first is not None else _p(None), _p(ab), _p(out),
+                                             _code(out, "out"), n_entries, width, int(blocks), int(taps), _stream()),
+           "rglru_scan")
+    return out
 
 
 SPLIT_MAX_VOCAB = 262144       # the largest vocabulary whose rows ``sample_packed(split=True)`` cuts into parts

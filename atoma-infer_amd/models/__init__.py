@@ -1,5 +1,5 @@
 """Architectures: builders from a typed configuration to a ModelSpec, and the model that runs one."""
-from . import llama, morulix, rakuvik, somesun  # register the architectures
+from . import bafilorn, llama, morulix, rakuvik, somesun  # register the architectures
 from .model import Model, load_model, random_model
 from .spec import LayerCall, ModelSpec
 

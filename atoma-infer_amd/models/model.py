@@ -47,8 +47,14 @@ class Model:
         readers = [b.entry_norm() for b in blocks[1:]]
         readers.append(spec.final_norm[1] if getattr(ctx, "wants_all_rows", False) else None)
         first = blocks[0].entry_norm() if blocks else None
-        resid, pending = spec.embedding[1].forward(ctx.tokens, first) if first is not None else \
-            (spec.embedding[1].forward(ctx.tokens), None)
+        if getattr(spec.embedding[1], "reads_context", False):
+            # an embedding that reads more of the step than its tokens (positions, entries, a state of its own)
+            from ..cache.pool import EMBEDDING_CALL
+            resid, pending = spec.embedding[1].forward_step(ctx, ctx.layer_cache(EMBEDDING_CALL)), None
+        elif first is not None:
+            resid, pending = spec.embedding[1].forward(ctx.tokens, first)
+        else:
+            resid, pending = spec.embedding[1].forward(ctx.tokens), None
         # a block that maps the stream from the embedding's rows too gets them as they were (gathered once more: the
         # stream's own rows are summed into in place), and one that is run several times is told which run this is
         embedded = spec.embedding[1].forward(ctx.tokens) if any(getattr(b, "reads_embedding", False) for b in blocks) \

@@ -489,7 +489,223 @@ class DifferentialAttention(PagedAttention):
         return linear_delta(y, self.w_o, None, self.w_o_tiled)
 
 
+def rotation_frequencies(base: float, dims: int, scaling: Optional[dict] = None):
+    """(float32 tensor [dims / 2] of base^(-2i / dims), worked out in double precision and rounded once; the factor on
+    cosines and sines).  ``scaling`` = {factor, original, fast, slow} slows the long waves down: with
+    where(t) = dims ln(original / (2 pi t)) / (2 ln base), lo = max(floor(where(fast)), 0), hi = min(ceil(where(slow)),
+    dims - 1) and ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i turns at
+    f_i / factor * ramp_i + f_i (1 - ramp_i), and cosines and sines are multiplied by 0.1 ln(factor) + 1."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / max(dims, 1))
+    mag = 1.0
+    if scaling is not None:
+        factor, original = float(scaling["factor"]), float(scaling["original"])
+
+        def where(turns: float) -> float:
+            return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+        lo = max(math.floor(where(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(where(float(scaling["slow"]))), dims - 1)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    return f.to(torch.float32), mag
+
+
+class GatedTiedValueAttention(PagedAttention):
+    """Attention whose values are its keys as projected (with their bias, before the rotation; no value projection),
+    with an output gate per column:
+
+    * q = W_q x + b_q, k = W_k x + b_k; grouped heads (query head h reads key head h // (heads / kv_heads));
+    * the first ``rotary_dim`` columns of every q and k head are rotated in half-split pairs (i, i + rotary_dim / 2),
+      or neighbouring ones with ``interleaved``, by position * frequency_i, the frequencies optionally slowed down band
+      by band (``rotary_scaling``, see ``rotation_frequencies``); angles are float32, worked out from the position;
+    * optional chunks or a window; with ``unit_sink`` the softmax denominator holds one more term exp(0) = 1;
+    * the heads' outputs are multiplied column by column with sigmoid(W_g x), then W_o x + b_o.
+
+    The output bias is not added here: ``out_bias`` (float32 [width] or None) is for whoever sums the output into the
+    stream or norms it.  Head sizes that are no multiple of 16 run as the next multiple (zero columns).
+
+    Tensors ([out, in]): ``q``, ``k``, ``g`` [heads * head_size, width], ``o``; with ``bias`` also ``q.b``, ``k.b``,
+    ``o.b``.
+    """
+
+    def __init__(self, width: int, num_heads: int, num_kv_heads: int, head_size: int, scale: float,
+                 rotary_base: float = 10000.0, rotary_dim: int = 0, rotary_scaling: Optional[dict] = None,
+                 interleaved: bool = False, chunk: Optional[int] = None, window: Optional[int] = None,
+                 unit_sink: bool = True, bias: bool = True):
+        padded = -(-int(head_size) // 16) * 16
+        super().__init__(width, num_heads, num_kv_heads, padded, None, window, scale, chunk)
+        self.hd_in = self.vd_in = int(head_size)
+        if rotary_dim % 2 or not 0 <= rotary_dim <= head_size or rotary_dim > 256:
+            raise ValueError(f"rotary_dim {rotary_dim} must be even, at most the head size {head_size} and at most 256")
+        self.rotary_base, self.rotary_dim, self.rotary_scaling = float(rotary_base), int(rotary_dim), rotary_scaling
+        self.interleaved, self.unit_sink, self.bias = bool(interleaved), bool(unit_sink), bool(bias)
+        nq, nk = self.nh * self.hd_in, self.nkv * self.hd_in
+        self.off_k, self.off_g = nq, nq + nk
+        self.w_in = self.b_q = self.b_k = self.out_bias = self.freq = None
+        self.mag = 1.0
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        q, kv, w = self.nh * self.hd_in, self.nkv * self.hd_in, self.width
+        specs = {"q": WeightSpec((q, w)), "k": WeightSpec((kv, w)), "g": WeightSpec((q, w)), "o": WeightSpec((w, q))}
+        if self.bias:
+            specs.update({"q.b": WeightSpec((q,), std=0.1), "k.b": WeightSpec((kv,), std=0.1),
+                          "o.b": WeightSpec((w,), std=0.1)})
+        return specs
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("q"), get("k"), get("g")]
+        dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        rows = sum(w.shape[0] for w in ws)
+        parts = [w.to(device=device, dtype=dt) for w in ws]
+        if (-rows) % 64:      # whole tiles for the matrix-core products
+            parts.append(torch.zeros(((-rows) % 64, self.width), dtype=dt, device=device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        if self.bias:
+            self.b_q, self.b_k = get("q.b").to(**f32).contiguous(), get("k.b").to(**f32).contiguous()
+            self.out_bias = get("o.b").to(**f32).contiguous()
+        freq, self.mag = rotation_frequencies(self.rotary_base, self.rotary_dim, self.rotary_scaling)
+        self.freq = freq.to(device).contiguous()
+        self.sinks = torch.zeros(self.nh, **f32) if self.unit_sink else None
+        self.act_dtype = act_dtype
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_o))
+
+    accepts_begun = False
+    takes_sink = False
+
+    def forward(self, x, ctx, cache, sink=None):
+        if not cache.writable:
+            raise NotImplementedError("tied-value attention reads only a cache of its own")
+        t = x.shape[0]
+        # the projection leaves in float32: biases, rotation and gates are float32 work
+        proj = linear(x, self.w_in, torch.float32)
+        q, gate = ops.tied_rope_prepare(proj, (0, self.off_k, self.off_g), self.b_q, self.b_k, ctx.positions, self.freq,
+                                        self.rotary_dim, self.interleaved, self.mag, cache.k, cache.v,
+                                        cache.slot_mapping, cache.page_size, self.nh, self.nkv, self.hd_in, self.hd,
+                                        x.dtype)
+        att = torch.empty((t, self.nh * self.hd), dtype=x.dtype, device=x.device)
+        self.attend(q, cache.k, cache.v, att, ctx, cache)
+        y = ops.gate_mul(att, gate, self.nh, self.hd_in, self.hd)
+        return linear_delta(y, self.w_o, None, self.w_o_tiled)
+
+
+class RotaryLatentAttention(PagedAttention):
+    """Attention over one cached latent vector per token, with queries through a latent of their own and a rotated key
+    part that all heads share:
+
+    * cq = norm(W_dq x) (``q_rank`` numbers, plain weight ``dq.norm``), q = W_uq cq: per head ``head_size`` columns
+      that meet the latent's keys and ``rotary_size`` columns that are rotated;
+    * W_dkv x has ``rank`` + ``rotary_size`` rows: the first ``rank``, normed with the plain weight ``dkv.norm``, are
+      the latent c; the rest, rotated, is a key part of its own.  Per head k = [W_uk c | that part], v = W_uv c
+      (``value_size`` columns); the cache keeps c and the rotated part, nothing else;
+    * rotation of neighbouring pairs (2i, 2i + 1) of the first ``rotary_dim`` of the ``rotary_size`` columns by
+      position * base^(-2i / rotary_dim), angles in float32 from the position;
+    * every earlier key is seen, ordinary softmax, the scale given; the heads' outputs are multiplied column by column
+      with sigmoid(W_g x), then W_o.
+
+    As in ``LatentAttention`` the heads' key and value maps act on the query's side: the attention kernels run with
+    one shared key head [c | rotated part] of ``rank + rotary_size`` columns (rounded up to a multiple of 16) against
+    queries [W_uk^T q_h | rotated q_h], and values [c | 0] of the same width.
+
+    Tensors ([out, in]): ``dq`` [q_rank, width], ``dq.norm``, ``uq`` [heads (head_size + rotary_size), q_rank], ``dkv``
+    [rank + rotary_size, width], ``dkv.norm`` [rank], ``uk`` [heads head_size, rank], ``uv`` [heads value_size, rank],
+    ``g`` [heads value_size, width], ``o`` [width, heads value_size].
+    """
+
+    def __init__(self, width: int, num_heads: int, head_size: int, rotary_size: int, value_size: int, rank: int,
+                 q_rank: int, scale: float, norm_eps: float, rotary_base: float = 10000.0,
+                 rotary_dim: Optional[int] = None):
+        wide = -(-(int(rank) + int(rotary_size)) // 16) * 16
+        super().__init__(width, num_heads, 1, wide, None, None, scale, None)
+        self.qd, self.rd, self.vd, self.rank, self.q_rank = int(head_size), int(rotary_size), int(value_size),             int(rank), int(q_rank)
+        self.rot = self.rd if rotary_dim is None else int(rotary_dim)
+        if self.rot % 2 or not 0 <= self.rot <= self.rd or self.rot > 256:
+            raise ValueError(f"rotary_dim {self.rot} must be even, at most rotary_size {self.rd} and at most 256")
+        self.hd_in = self.vd_in = wide
+        self.norm_eps, self.rotary_base = float(norm_eps), float(rotary_base)
+        self.off_c = self.q_rank
+        self.off_g = self.off_c + self.rank + self.rd
+        self.w_in = self.w_uq = self.w_uk = self.w_uv = self.q_norm = self.c_norm = self.freq = None
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        h, w, r, qr = self.nh, self.width, self.rank, self.q_rank
+        return {"dq": WeightSpec((qr, w)), "dq.norm": WeightSpec((qr,), "norm"),
+                "uq": WeightSpec((h * (self.qd + self.rd), qr), std=qr ** -0.5),
+                "dkv": WeightSpec((r + self.rd, w)), "dkv.norm": WeightSpec((r,), "norm"),
+                "uk": WeightSpec((h * self.qd, r), std=r ** -0.5), "uv": WeightSpec((h * self.vd, r), std=r ** -0.5),
+                "g": WeightSpec((h * self.vd, w)), "o": WeightSpec((w, h * self.vd))}
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("dq"), get("dkv"), get("g")]
+        dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        rows = sum(w.shape[0] for w in ws)
+        parts = [w.to(device=device, dtype=dt) for w in ws]
+        if (-rows) % 64:      # whole tiles for the matrix-core products
+            parts.append(torch.zeros(((-rows) % 64, self.width), dtype=dt, device=device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_uq = get("uq").to(device).contiguous()
+        # per head [out, in]: on the query's side the key map transposed beside an identity that hands the rotated
+        # columns through, zero rows up to the cache's width; the value map with zero columns behind the latent's
+        uk = get("uk").to(device).view(self.nh, self.qd, self.rank).transpose(1, 2)            # [h, rank, qd]
+        wq = torch.zeros((self.nh, self.hd, self.qd + self.rd), dtype=uk.dtype, device=device)
+        wq[:, : self.rank, : self.qd] = uk
+        wq[:, self.rank: self.rank + self.rd, self.qd:] = torch.eye(self.rd, dtype=uk.dtype, device=device)
+        self.w_uk = wq.contiguous()
+        uv = get("uv").to(device).view(self.nh, self.vd, self.rank)
+        self.w_uv = torch.nn.functional.pad(uv, (0, self.hd - self.rank)).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        self.q_norm, self.c_norm = get("dq.norm").to(**f32).contiguous(), get("dkv.norm").to(**f32).contiguous()
+        self.freq = rotation_frequencies(self.rotary_base, self.rot)[0].to(device).contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        self.act_dtype = act_dtype
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_uq, self.w_uk, self.w_uv, self.w_o))
+
+    accepts_begun = False
+    takes_sink = False
+
+    def forward(self, x, ctx, cache, sink=None):
+        if not cache.writable:
+            raise NotImplementedError("latent attention reads only a cache of its own")
+        t = x.shape[0]
+        # both latents and the gates leave their product in float32: norms, rotation and gates are float32 work
+        proj = linear(x, self.w_in, torch.float32)
+        cq, gate = ops.latent_rope_prepare(proj, (0, self.off_c, self.off_g), self.q_rank, self.rank, self.rd, self.hd,
+                                           self.nh * self.vd, self.q_norm, self.c_norm, self.norm_eps, ctx.positions,
+                                           self.freq, self.rot, cache.k, cache.v, cache.slot_mapping, cache.page_size,
+                                           x.dtype)
+        q = ops.latent_q_rope(linear(cq, self.w_uq, torch.float32), ctx.positions, self.freq, self.rot, self.nh,
+                              self.qd, self.rd, x.dtype)
+        ql = ops.head_linear(q, self.w_uk, x.dtype)                      # the queries in the cached key's columns
+        mixed = torch.empty((t, self.nh * self.hd), dtype=x.dtype, device=proj.device)
+        self.attend(ql, cache.k, cache.v, mixed, ctx, cache)
+        out = ops.head_linear(mixed, self.w_uv, x.dtype, gate)           # the heads' values, gated column by column
+        return linear_delta(out, self.w_o, sink, self.w_o_tiled)
+
+
 register_mixer("latent_attention", LatentAttention)
 register_mixer("differential_attention", DifferentialAttention)
 register_mixer("attention", PagedAttention)
 register_mixer("tied_value_attention", TiedValueAttention)
+register_mixer("gated_tied_value_attention", GatedTiedValueAttention)
+register_mixer("rotary_latent_attention", RotaryLatentAttention)

@@ -75,4 +75,39 @@ class SwiGLU(FeedForward):
         return linear_delta(h, self.w_down, sink, self.w_down_tiled)
 
 
+class DenseFeedForward(FeedForward):
+    """A feed-forward without a gate: ``down(act(up(x)))``, no biases; ``activation`` "relu2" is the square of relu."""
+
+    def __init__(self, width: int, intermediate: int, names=("up", "down"), activation: str = "relu2"):
+        if activation != "relu2":
+            raise ValueError(f"activation {activation!r} is not supported (known: relu2)")
+        self.width, self.inter, self.names, self.activation = int(width), int(intermediate), tuple(names), activation
+        self.w_up = self.w_down = self.w_up_tiled = self.w_down_tiled = None
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        return {self.names[0]: WeightSpec((self.inter, self.width)), self.names[1]: WeightSpec((self.width, self.inter))}
+
+    def load(self, get, device, act_dtype) -> None:
+        self.w_up = get(self.names[0]).to(device).contiguous()
+        self.w_down = get(self.names[1]).to(device).contiguous()
+        self.w_up_tiled = self.w_down_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_up.dtype is torch.bfloat16 and self.w_down.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            plan = gemm_bf16.tiled_plan(self.inter, self.width, swiglu=False)
+            if plan is not None:
+                self.w_up_tiled = gemm_bf16.tile_weight(self.w_up, *plan)
+            self.w_down_tiled = gemm_bf16.tile_copies_resid(self.w_down)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_up, self.w_down))
+
+    def forward(self, x, ctx, sink=None):
+        u = linear(x, self.w_up, tiled=self.w_up_tiled)
+        return linear_delta(ops.dense_act(u, x.dtype, self.activation), self.w_down, sink, self.w_down_tiled)
+
+
 register_feed_forward("swiglu", SwiGLU)
+register_feed_forward("dense", DenseFeedForward)

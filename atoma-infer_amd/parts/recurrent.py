@@ -290,6 +290,168 @@ class MinGRU(Mixer):
         return linear_delta(y, self.w_o, None, self.w_o_tiled)
 
 
+class LightningAttention(Mixer):
+    """Linear attention with one fixed decay per head: q = silu(W_q x), k = silu(W_k x) (``heads`` x ``dim``),
+    v = silu(W_v x) (``heads`` x ``vdim``); per head
+
+        S <- decay_h S + k v^T;   o = S^T q      (no other scale),
+
+    the heads' outputs normed together (RMS, plain weight ``norm``), multiplied by sigmoid(W_g x) and projected by W_o.
+    A request's state is S, float32 [heads][vdim][dim], zero at its start.  The four input projections are one product
+    with float32 sums that leaves unrounded; SiLU, the recurrence, the norm and the gate are float32 in both dtypes.
+
+    Tensors ([out, in]): ``q``, ``k`` [heads dim, width], ``v``, ``g`` [heads vdim, width], ``norm`` [heads vdim],
+    ``o`` [width, heads vdim].
+    """
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, norm_eps: float):
+        decay = [float(d) for d in decay]
+        if len(decay) != heads:
+            raise ValueError(f"{len(decay)} decays for {heads} heads")
+        if dim > 256:
+            raise ValueError("key sizes beyond 256 are not supported by the recurrence's kernel")
+        self.width, self.heads, self.dim, self.vdim, self.decay_list = int(width), int(heads), int(dim), int(vdim), decay
+        self.norm_eps = float(norm_eps)
+        nq, nv = self.heads * self.dim, self.heads * self.vdim
+        self.off_k, self.off_v, self.off_g = nq, 2 * nq, 2 * nq + nv
+        self.w_in = self.w_o = self.w_o_tiled = self.norm_w = self.decay = None
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        w, nq, nv = self.width, self.heads * self.dim, self.heads * self.vdim
+        return {"q": WeightSpec((nq, w), std=0.08), "k": WeightSpec((nq, w), std=0.08),
+                "v": WeightSpec((nv, w), std=0.08), "g": WeightSpec((nv, w), std=0.08),
+                "norm": WeightSpec((nv,), "norm"), "o": WeightSpec((w, nv))}
+
+    def state_spec(self) -> StateSpec:
+        return StateSpec((self.heads * self.vdim * self.dim,), "float32")
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("q"), get("k"), get("v"), get("g")]
+        dt = ws[0].dtype if all(w.dtype is ws[0].dtype for w in ws) else torch.float32
+        rows = sum(w.shape[0] for w in ws)
+        parts = [w.to(device=device, dtype=dt) for w in ws]
+        if (-rows) % 64:      # whole tiles for the matrix-core products
+            parts.append(torch.zeros(((-rows) % 64, self.width), dtype=dt, device=device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        self.norm_w = get("norm").to(**f32).contiguous()
+        self.decay = torch.tensor(self.decay_list, dtype=torch.float64).to(**f32).contiguous()
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_o))
+
+    def forward(self, x, ctx, cache):
+        proj = linear(x, self.w_in, torch.float32)
+        o = ops.lightning_scan(proj, (0, self.off_k, self.off_v), ctx.q_start, ctx.state_slots, cache.state, self.decay,
+                               self.heads, self.dim, self.vdim)
+        y = ops.lightning_out(o, proj, self.off_g, self.norm_w, self.norm_eps, x.dtype)
+        return linear_delta(y, self.w_o, None, self.w_o_tiled)
+
+
+class GatedLinearRecurrence(Mixer):
+    """Griffin's recurrent block around a real-gated linear recurrent unit, ``inner`` channels:
+
+        g = gelu_tanh(W_y x + b_y);   u = conv(W_x x + b_x)     (causal, per channel, ``taps`` taps, bias, no activation)
+        r = sigmoid(Ra u + ba);   i = sigmoid(Ri u + bi)        (Ra, Ri: ``blocks`` square blocks on the diagonal)
+        a = exp(-8 r softplus(lam));   S <- a S + sqrt(1 - a^2) i u;   out = W_o (S g).
+
+    A request's state is the convolution's last ``taps - 1`` inputs and S, float32, zero at its start.  The two input
+    projections are one product with float32 sums that leaves unrounded; everything behind it, the gates' products
+    included, is float32 in both dtypes.  The step is linear in S, so entries of many tokens are walked in stretches
+    side by side (the plan of ``ops.mingru_plan``), decoded tokens by the plain walk.
+
+    Tensors ([out, in]): ``y``, ``x`` [inner, width] with ``y.b``, ``x.b``; ``conv`` [inner, taps] (last column: the
+    current token), ``conv.b``; ``ra``, ``ri`` [blocks, inner / blocks, inner / blocks] with ``ra.b``, ``ri.b``
+    [blocks, inner / blocks]; ``lam`` [inner]; ``o`` [width, inner].
+    """
+
+    def __init__(self, width: int, inner: int, blocks: int, taps: int):
+        if inner <= 0 or blocks <= 0 or inner % blocks or not 1 <= taps <= 64:
+            raise ValueError(f"a recurrence of {inner} channels in {blocks} blocks with {taps} taps is not supported")
+        self.width, self.inner, self.blocks, self.taps = int(width), int(inner), int(blocks), int(taps)
+        self.bs = self.inner // self.blocks
+        self.w_in = self.w_gates = self.w_o = self.w_o_tiled = None
+        self.b_y = self.b_x = self.conv = self.conv_b = self.b_a = self.b_i = self.sp = None
+        self.out_bias = None
+
+    def graph_safe(self) -> bool:
+        return True
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        w, n, b, bs, k = self.width, self.inner, self.blocks, self.bs, self.taps
+        return {"y": WeightSpec((n, w), std=0.08), "y.b": WeightSpec((n,), std=0.3),
+                "x": WeightSpec((n, w), std=0.08), "x.b": WeightSpec((n,), std=0.3),
+                "conv": WeightSpec((n, k), std=0.4), "conv.b": WeightSpec((n,), std=0.1),
+                "ra": WeightSpec((b, bs, bs), std=bs ** -0.5), "ra.b": WeightSpec((b, bs), std=0.5),
+                "ri": WeightSpec((b, bs, bs), std=bs ** -0.5), "ri.b": WeightSpec((b, bs), std=0.5),
+                "lam": WeightSpec((n,), std=1.0, mean=-1.0), "o": WeightSpec((w, n))}
+
+    def state_spec(self) -> StateSpec:
+        return StateSpec((self.taps * self.inner,), "float32")
+
+    def load(self, get, device, act_dtype) -> None:
+        ws = [get("y"), get("x")]
+        dt = ws[0].dtype if ws[0].dtype is ws[1].dtype else torch.float32
+        parts = [w.to(device=device, dtype=dt) for w in ws]
+        if (-2 * self.inner) % 64:      # whole tiles for the matrix-core products
+            parts.append(torch.zeros(((-2 * self.inner) % 64, self.width), dtype=dt, device=device))
+        self.w_in = torch.cat(parts, dim=0).contiguous()
+        self.w_o = get("o").to(device).contiguous()
+        f32 = dict(device=device, dtype=torch.float32)
+        vec = lambda name: get(name).to(**f32).reshape(-1).contiguous()
+        self.b_y, self.b_x, self.conv_b = vec("y.b"), vec("x.b"), vec("conv.b")
+        self.conv = get("conv").to(**f32).contiguous()
+        self.b_a, self.b_i = vec("ra.b"), vec("ri.b")
+        # per block the rows of Ra, then those of Ri: one product per block gives [r | i] before their biases
+        self.w_gates = torch.cat([get("ra").to(**f32), get("ri").to(**f32)], dim=1).contiguous()
+        # softplus(lam) in float32, once: log(1 + exp(lam)) in its stable form
+        lam = vec("lam")
+        self.sp = (torch.clamp(lam, min=0.0) + torch.log1p(torch.exp(-lam.abs()))).contiguous()
+        self.w_o_tiled = None
+        if act_dtype is torch.bfloat16 and self.w_o.dtype is torch.bfloat16:
+            from ..kernels import gemm_bf16
+            self.w_o_tiled = gemm_bf16.tile_copies_resid(self.w_o)
+
+    def device_bytes(self) -> int:
+        return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_gates, self.w_o))
+
+    def _plan_key(self):
+        return ("mingru_stretches", -(-self.inner // 256))
+
+    def step_planner(self, page_size: int, cache_dtype: torch.dtype):
+        import numpy as np
+        cus = torch.cuda.get_device_properties(self.w_o.device).multi_processor_count
+
+        def plan(starts, counts, bucket):
+            got = ops.mingru_plan(counts, self.inner, cus)
+            return got if got is not None else (np.zeros(0, dtype=np.int32), 0)
+        return self._plan_key(), plan
+
+    def forward(self, x, ctx, cache):
+        proj = linear(x, self.w_in, torch.float32)
+        u, g = ops.rglru_conv(proj, 0, self.inner, self.b_y, self.b_x, self.conv, self.conv_b, ctx.token_seq,
+                              ctx.q_start, ctx.state_slots, cache.state, self.inner, self.taps)
+        gates = ops.head_linear(u, self.w_gates, torch.float32)
+        plan = getattr(ctx, "plans", {}).get(self._plan_key())
+        if plan is None and getattr(ctx, "h_counts", None) is not None:
+            got = ops.mingru_plan(ctx.h_counts, self.inner)      # a caller without a step planner: plan here and now
+            if got is not None:
+                plan = (torch.from_numpy(got[0]).to(x.device), got[1])
+        y = ops.rglru_scan(gates, u, g, self.b_a, self.b_i, self.sp, ctx.q_start, ctx.state_slots, cache.state,
+                           self.blocks, self.taps, x.dtype, plan)
+        return linear_delta(y, self.w_o, None, self.w_o_tiled)
+
+
 register_mixer("gated_delta_rule", GatedDeltaRule)
 register_mixer("mingru", MinGRU)
+register_mixer("lightning_attention", LightningAttention)
+register_mixer("gated_linear_recurrence", GatedLinearRecurrence)
 register_mixer("state_space_duality", StateSpaceDuality)

@@ -45,6 +45,9 @@ def random_tensor(name: str, ws: WeightSpec, seed: int, dtype: torch.dtype, norm
     elif ws.init == "tail_heavy":      # weights of a sum whose last term carries most: N(mean, std), the last + 0.7
         t = torch.randn(ws.drawn_shape, generator=g, dtype=torch.float32) * ws.std + ws.mean
         t.view(-1)[-1] += 0.7
+    elif ws.init == "near_identity":   # a square matrix that mixes a little: the identity + N(0, std)
+        t = torch.eye(ws.drawn_shape[0], dtype=torch.float32) + \
+            torch.randn(ws.drawn_shape, generator=g, dtype=torch.float32) * ws.std
     elif ws.init == "int_table":
         return torch.randint(0, max(ws.high, 1), ws.drawn_shape, generator=g, dtype=torch.int32)
     else:
