@@ -76,8 +76,10 @@ __device__ __forceinline__ Step step_of(const float* __restrict__ gates, int ldg
   const int blk = c / bs, k = c % bs;
   const float* gr = gates + (size_t)t * ldg + (size_t)blk * 2 * bs;
   const float r = sigm(gr[k] + bra), i = sigm(gr[bs + k] + bri);
-  const float a = expf(-8.0f * r * sp);
-  return Step{a, sqrtf(1.0f - a * a) * i * u[(size_t)t * width + c]};
+  // 1 - a^2 = -expm1(2 log a): exact also where a is close to one
+  const float la = -8.0f * r * sp;
+  const float a = expf(la);
+  return Step{a, sqrtf(-expm1f(2.0f * la)) * i * u[(size_t)t * width + c]};
 }
 
 template <typename TO>

@@ -31,12 +31,14 @@ class WeightSpec:
 
     ``init``: "linear" and "embedding" draw N(mean, std), by default N(0, 0.02); "norm" is 1 (plus N(0, norm_jitter)
     on request); "int_table" draws integers in [0, high).  Integer tables are kept as int32 on the device.
+    ``optional``: a checkpoint may lack the tensor (``get`` then raises KeyError and the part takes its default).
     """
     shape: Tuple[int, ...]
     init: str = "linear"
     high: int = 0
     mean: float = 0.0
     std: float = 0.02
+    optional: bool = False
 
     @property
     def is_int(self) -> bool:

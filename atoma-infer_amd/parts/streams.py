@@ -50,18 +50,25 @@ class StreamWeights(Part):
         if self.copies is None:
             return {}
         s = self.copies
-        return {f"{self.prefix}.in": WeightSpec((s,), "linear", mean=1.0 / s, std=0.1),
-                f"{self.prefix}.out": WeightSpec((s,), "linear", mean=1.0, std=0.2),
-                f"{self.prefix}.mix": WeightSpec((s, s), "near_identity", std=0.1)}
+        # (a checkpoint of one copy may come without them: they are then one, the plain residual)
+        opt = s == 1
+        return {f"{self.prefix}.in": WeightSpec((s,), "linear", mean=1.0 / s, std=0.1, optional=opt),
+                f"{self.prefix}.out": WeightSpec((s,), "linear", mean=1.0, std=0.2, optional=opt),
+                f"{self.prefix}.mix": WeightSpec((s, s), "near_identity", std=0.1, optional=opt)}
 
     def load(self, get, device, act_dtype) -> None:
         f32 = dict(device=device, dtype=torch.float32)
         if self.copies is None:
             self.w_in = self.mix = self.out = torch.ones(1, **f32)
             return
-        self.w_in = get(f"{self.prefix}.in").to(**f32).contiguous()
-        self.mix = get(f"{self.prefix}.mix").to(**f32).contiguous()
-        self.out = get(f"{self.prefix}.out").to(**f32).contiguous()
+        def take(name, shape):
+            try:
+                return get(f"{self.prefix}.{name}").to(**f32).contiguous()
+            except KeyError:
+                if self.copies != 1:
+                    raise
+                return torch.ones(shape, **f32)
+        self.w_in, self.mix, self.out = take("in", (1,)), take("mix", (1, 1)), take("out", (1,))
 
 
 class StreamBlock(Block):

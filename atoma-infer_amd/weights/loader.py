@@ -104,7 +104,7 @@ def check_checkpoint(spec, ckpt: Checkpoint) -> None:
     want = expected_tensors(spec)
     have = set(ckpt.names())
     ignorable = [re.compile(p) for p in spec.ignorable]
-    missing = [n for n in want if n not in have]
+    missing = [n for n, ws in want.items() if n not in have and not ws.optional]
     unexpected = sorted(n for n in have if n not in want and not any(r.fullmatch(n) for r in ignorable))
     wrong_shape, wrong_kind = [], []
     for n, ws in want.items():

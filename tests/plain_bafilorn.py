@@ -233,7 +233,8 @@ def forward(tokens, w, cfg):
     eps = cfg["norm"]["eps"]
     p = np.arange(len(tokens))
     x0 = embed(np.asarray(tokens), w, cfg)
-    s = int(cfg.get("streams", 1))
+    copies = cfg.get("streams")                 # absent: one stream and no connection tensors
+    s = int(copies or 1)
     xs = [x0.copy() for _ in range(s)]
     seen = []
     for li in run_order(cfg):
@@ -243,7 +244,7 @@ def forward(tokens, w, cfg):
         if layer.get("mlp") is not None:
             subs.append((2, lambda h: feed_forward(h, w, pre + "mlp.")))
         for q, fn in subs:
-            if s > 1:
+            if copies is not None:
                 hin, hmix, hout = w[pre + f"hc{q}.in"], w[pre + f"hc{q}.mix"], w[pre + f"hc{q}.out"]
                 u = sum(hin[i] * xs[i] for i in range(s))
                 y = fn(norm_one_plus(u, w[pre + f"norm{q}"], eps))
