@@ -299,10 +299,14 @@ class LightningAttention(Mixer):
     the heads' outputs normed together (RMS, plain weight ``norm``), multiplied by sigmoid(W_g x) and projected by W_o.
     A request's state is S, float32 [heads][vdim][dim], zero at its start.  The four input projections are one product
     with float32 sums that leaves unrounded; SiLU, the recurrence, the norm and the gate are float32 in both dtypes.
+    With bfloat16 activations, entries of ``CHUNKED_FROM`` tokens or more run 64 tokens at a time on the matrix cores,
+    q, k and v rounded to bfloat16 there (as activations are), the state and every sum still float32.
 
     Tensors ([out, in]): ``q``, ``k`` [heads dim, width], ``v``, ``g`` [heads vdim, width], ``norm`` [heads vdim],
     ``o`` [width, heads vdim].
     """
+
+    CHUNKED_FROM = 24
 
     def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, norm_eps: float):
         decay = [float(d) for d in decay]
@@ -350,8 +354,10 @@ class LightningAttention(Mixer):
 
     def forward(self, x, ctx, cache):
         proj = linear(x, self.w_in, torch.float32)
+        chunked = self.CHUNKED_FROM if (x.dtype is torch.bfloat16 and self.dim % 32 == 0 and self.dim <= 128
+                                        and min(self.decay_list) > 0.0) else 0
         o = ops.lightning_scan(proj, (0, self.off_k, self.off_v), ctx.q_start, ctx.state_slots, cache.state, self.decay,
-                               self.heads, self.dim, self.vdim)
+                               self.heads, self.dim, self.vdim, chunked)
         y = ops.lightning_out(o, proj, self.off_g, self.norm_w, self.norm_eps, x.dtype)
         return linear_delta(y, self.w_o, None, self.w_o_tiled)
 

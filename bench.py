@@ -19,7 +19,10 @@ width: prefill of 2,048 tokens and decode steps at batch 1, 8 and 64 through the
 ``--compare morulix`` does the same for the Morulix decoder (latent attention, a state-space recurrence and windowed
 attention in turn, each beside a dense feed-forward, behind one pass of its loop's entry), and ``--compare rakuvik``
 for the Rakuvik decoder (differential attention and a minGRU recurrence in turn, dense and routed feed-forwards in
-turn, the layers' results averaged over depth).
+turn, the layers' results averaged over depth).  ``--compare bafilorn`` measures the Bafilorn decoder (a stream in
+four copies behind an embedding of token pairs; latent attention with a rotated key part, lightning attention, and
+chunked attention with tied values beside a gated linear recurrence in turn, each before a dense feed-forward with the
+square of relu) beside the Morulix of equal sizes, the closest of the other designs, and the Llama.
 
 ``--workload`` runs one of the other two workloads instead and prints ONE line of its own:
 ``serve3b``: Llama-3.2-3B sizes, 64 requests with prompt lengths uniform in [128, 4096] (seeded), 256 generated tokens
@@ -309,6 +312,56 @@ def step_bytes_rakuvik(model, cfg: dict, batch: int, ctx: float) -> float:
     return total
 
 
+def bafilorn_like(llama: dict, layers: int) -> dict:
+    """The Bafilorn configuration beside ``llama`` and ``morulix_like(llama)``: the same width and vocabulary; four
+    copies of the stream; a table of 65,521 token pairs; layers in turn latent attention (half as many heads of twice
+    the size, 32 of their columns rotated, over a cached key of the Morulix's latent width, queries through a latent of
+    half the model's width), lightning attention (as many heads as the Llama, keys and values of 128 columns: a state
+    as large as the Morulix recurrence's), chunked attention with the Llama's heads and tied values beside a gated
+    linear recurrence of the model's width in 16 blocks, and lightning attention again; feed-forwards of one and a half
+    times the Llama's width (two matrices where the gated one has three)."""
+    w, nh, nkv = llama["hidden_size"], llama["num_attention_heads"], llama["num_key_value_heads"]
+    hd = w // nh
+    mlp = {"kind": "dense", "ff": 3 * llama["intermediate_size"] // 2}
+    wide = 128 if w < 3072 else 256
+    lat = {"type": "latent_attention", "mlp": mlp,
+           "mixer": {"dim": 2 * hd - 32, "heads": nh // 2, "kv_rank": wide - 32 if wide == 256 else wide, "q_rank": w // 2,
+                     "rot_dim": 32, "rot": {"base": 10000.0, "dims": 32}, "scale": (2 * hd) ** -0.5, "vdim": 2 * hd}}
+    lit = {"type": "lightning", "mlp": mlp,
+           "mixer": {"decay": [1.0 - 2.0 ** (-3.0 - 5.0 * h / nh) for h in range(nh)], "dim": 128, "heads": nh, "vdim": 128}}
+    par = {"type": "parallel", "mlp": mlp,
+           "mixer": {"left": {"dim": hd, "heads": nh, "kv_heads": nkv, "vdim": hd, "scale": hd ** -0.5,
+                              "mask": {"size": 1024},
+                              "rot": {"base": llama["rope_theta"], "dims": hd,
+                                      "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+                     "right": {"blocks": 16, "conv": 4, "width": w}}}
+    kinds = [lat, lit, par, lit]
+    return {"architecture": "Bafilorn", "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}},
+            "layers": [kinds[i % 4] for i in range(layers)], "norm": {"eps": 1e-5}, "streams": 4,
+            "loop": {"start": 0, "stop": layers, "times": 1}, "vocab": llama["vocab_size"], "width": w,
+            "max_positions": llama["max_position_embeddings"]}
+
+
+def step_bytes_bafilorn(model, cfg: dict, batch: int, ctx: float) -> float:
+    """Bytes a decode step of ``batch`` requests at context ``ctx`` has to read (and, for the states, write): every
+    matrix once, each request's cached keys and values of the latent layers (both as wide as the key), the keys and
+    values of its current chunk, the recurrent states twice, the copies of the stream twice per sublayer."""
+    total = float(model.weight_bytes())
+    w, copies = cfg["width"], cfg.get("streams") or 1
+    for l in cfg["layers"]:
+        m = l["mixer"]
+        if l["type"] == "latent_attention":
+            total += batch * ctx * 2.0 * 2 * (-(-(m["kv_rank"] + m["rot_dim"]) // 16) * 16)
+        elif l["type"] == "lightning":
+            total += batch * 2 * 4.0 * m["heads"] * m["dim"] * m["vdim"]
+        else:
+            a, r = m["left"], m["right"]
+            seen = min(ctx, a["mask"]["size"] / 2.0) if a.get("mask") else ctx
+            total += batch * (2.0 * 2 * a["kv_heads"] * a["dim"] * seen + 2 * 4.0 * r["conv"] * r["width"])
+        total += batch * 4.0 * w * copies * 2 * (2 if l["mlp"] else 1)
+    return total
+
+
 def compare_main(args) -> int:
     import torch
     import atoma_infer_amd  # noqa: F401
@@ -318,9 +371,13 @@ def compare_main(args) -> int:
     layers = args.layers or 4
     llama = dict(dict(LLAMA_1B, **OTHER_SIZES.get(sizes, {})), num_hidden_layers=layers)
     design = args.compare
-    sun = {"somesun": somesun_like, "morulix": morulix_like, "rakuvik": rakuvik_like}[design](llama, layers)
+    sun = {"somesun": somesun_like, "morulix": morulix_like, "rakuvik": rakuvik_like,
+           "bafilorn": bafilorn_like}[design](llama, layers)
     out = {}
-    for name, cfg in (("llama", llama), (design, sun)):
+    pairs = [("llama", llama), (design, sun)]
+    if design == "bafilorn":      # also the closest of the other designs, at the same sizes
+        pairs.insert(1, ("morulix", morulix_like(llama, layers)))
+    for name, cfg in pairs:
         if args.only and args.only != name:
             continue
         log(f"{name}: building {layers} layers at {sizes} sizes (random weights) ...")
@@ -334,8 +391,10 @@ def compare_main(args) -> int:
             d, ctx = decode_run(model, b, args.prompt_len, st, min(args.warmup, 4), args.context)
             if name == "somesun":
                 nbytes = step_bytes_somesun(sun, b, ctx)
+            elif name == "bafilorn":
+                nbytes = step_bytes_bafilorn(model, sun, b, ctx)
             elif name == "morulix":
-                nbytes = step_bytes_morulix(model, sun, b, ctx)
+                nbytes = step_bytes_morulix(model, cfg, b, ctx)
             elif name == "rakuvik":
                 nbytes = step_bytes_rakuvik(model, sun, b, ctx)
             else:
@@ -420,9 +479,9 @@ def main() -> int:
     ap.add_argument("--top-p", type=float, default=1.0)
     ap.add_argument("--workload", choices=["decode", *WORKLOADS], default="decode",
                     help="decode: the default run; serve3b, long8b: the other two workloads, one line of their own")
-    ap.add_argument("--compare", choices=["somesun", "morulix", "rakuvik"], default=None,
+    ap.add_argument("--compare", choices=["somesun", "morulix", "rakuvik", "bafilorn"], default=None,
                     help="measure that design at --sizes (1b, 3b) beside the Llama of equal sizes, one line of its own")
-    ap.add_argument("--only", choices=["llama", "somesun", "morulix", "rakuvik"], default=None, help="with --compare: one of the two models")
+    ap.add_argument("--only", choices=["llama", "somesun", "morulix", "rakuvik", "bafilorn"], default=None, help="with --compare: one of the two models")
     ap.add_argument("--requests", type=int, default=0, help="requests of a --workload run (default: the workload's)")
     ap.add_argument("--no-peaks", action="store_true", help="skip the probes of what the GPU delivers")
     ap.add_argument("--chain-floors", action="store_true",

@@ -198,7 +198,8 @@ def _recurrent_case(part, hs, dtype, state_width):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads, dim, vdim", [(3, 16, 24), (1, 128, 64), (2, 10, 5), (1, 1, 1), (5, 200, 17), (2, 64, 32)])
+@pytest.mark.parametrize("heads, dim, vdim", [(3, 16, 24), (1, 128, 64), (2, 10, 5), (1, 1, 1), (5, 200, 17), (2, 64, 32),
+                                              (3, 32, 40), (2, 96, 16), (4, 128, 128)])
 def test_lightning_attention_alone_whole_and_in_portions(heads, dim, vdim, dtype):
     from atoma_infer_amd.parts import LightningAttention
     width = 64
