@@ -666,11 +666,41 @@ dense_act_kernel(const TI* __restrict__ u, int ld, TO* __restrict__ out, int int
   }
 }
 
+// eight bfloat16 values per thread (16-byte loads and stores); needs inter % 8 == 0, ld % 8 == 0 and aligned rows
+__global__ void __launch_bounds__(256)
+dense_act_vec8_kernel(const uint16_t* __restrict__ u, int ld, uint16_t* __restrict__ out, int inter, int n_tokens) {
+  const int octs = inter >> 3;
+  const size_t total = (size_t)n_tokens * octs;
+  for (size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (size_t)gridDim.x * 256) {
+    const size_t t = idx / octs;
+    const int i = (int)(idx % octs) * 8;
+    const uint4 raw = *reinterpret_cast<const uint4*>(u + t * ld + i);
+    const uint16_t* a = reinterpret_cast<const uint16_t*>(&raw);
+    uint4 oraw;
+    uint16_t* o = reinterpret_cast<uint16_t*>(&oraw);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float v = bf16_bits_to_f32(a[e]);
+      o[e] = f32_to_bf16_bits(v > 0.f ? v * v : 0.f);
+    }
+    *reinterpret_cast<uint4*>(out + t * inter + i) = oraw;
+  }
+}
+
 extern "C" int atoma_dense_act(const void* u, int u_dtype, int ld, void* out, int out_dtype, int n_tokens, int inter,
                                int act, hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (inter <= 0 || ld < inter || act != 0) return ATOMA_ERR_SHAPE;
   const size_t total = (size_t)n_tokens * inter;
+  if (u_dtype == kBF16 && out_dtype == kBF16 && inter % 8 == 0 && ld % 8 == 0 && ((uintptr_t)u & 15) == 0 &&
+      ((uintptr_t)out & 15) == 0) {
+    int vb = (int)((total / 8 + 255) / 256);
+    if (vb > 16384) vb = 16384;
+    hipLaunchKernelGGL(dense_act_vec8_kernel, dim3(vb), dim3(256), 0, stream, (const uint16_t*)u, ld, (uint16_t*)out,
+                       inter, n_tokens);
+    ATOMA_LAUNCH_CHECK();
+    return 0;
+  }
   int blocks = (int)((total + 255) / 256);
   if (blocks > 65536) blocks = 65536;
   if (u_dtype == kF32 && out_dtype == kF32)

@@ -114,8 +114,15 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 
 constexpr int kChunk = 64, kPad = 8, kCols = 32;
 
-__device__ __forceinline__ uint16_t hi_of(float x) { return f32_to_bf16_bits(x); }
-__device__ __forceinline__ uint16_t lo_of(float x, uint16_t hi) { return f32_to_bf16_bits(x - bf16_bits_to_f32(hi)); }
+// (the chunked kernel's conversions are the hardware's round-to-nearest-even ones, and its SiLU uses the fast
+// exponential and reciprocal: its results are rounded to bfloat16 at once)
+__device__ __forceinline__ uint16_t bf16_of(float x) {
+  const __bf16 b = static_cast<__bf16>(x);
+  return __builtin_bit_cast(uint16_t, b);
+}
+__device__ __forceinline__ float silu_fast(float x) { return x * __frcp_rn(1.0f + __expf(-x)); }
+__device__ __forceinline__ uint16_t hi_of(float x) { return bf16_of(x); }
+__device__ __forceinline__ uint16_t lo_of(float x, uint16_t hi) { return bf16_of(x - bf16_bits_to_f32(hi)); }
 __device__ __forceinline__ float pow_int(float l2, int n) { return n == 0 ? 1.0f : exp2f(l2 * (float)n); }
 __device__ __forceinline__ bf16x8 frag(const uint16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
@@ -165,31 +172,54 @@ lightning_chunk_kernel(const float* __restrict__ proj, int ld, int off_q, int of
         }
       }
   }
+  // A chunk's q, k, v are asked for a chunk ahead and wait in registers: 4 neighbouring columns of q and of k per
+  // load, DIM / 16 loads of each a thread, and 8 values of v.
+  constexpr int NQ = DIM / 16, NV = kChunk * kCols / 256, RT = DIM / 4;      // RT: threads a row of q
+  float4 rq[NQ], rk[NQ];
+  float rv[NV];
+  auto ask = [&](int tb, int n) {
+#pragma unroll
+    for (int it = 0; it < NQ; ++it) {
+      const int idx = threadIdx.x + 256 * it, j = idx / RT, c = (idx % RT) * 4;
+      const float* row = proj + (size_t)(tb + (j < n ? j : n - 1)) * ld + h * DIM + c;
+      rq[it] = *reinterpret_cast<const float4*>(row + off_q);
+      rk[it] = *reinterpret_cast<const float4*>(row + off_k);
+    }
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int idx = threadIdx.x + 256 * it, j = idx / kCols, v = idx % kCols;
+      rv[it] = v0 + v < vdim ? proj[(size_t)(tb + (j < n ? j : n - 1)) * ld + off_v + h * vdim + v0 + v] : 0.f;
+    }
+  };
+  ask(t0, t1 - t0 < kChunk ? t1 - t0 : kChunk);
   for (int tb = t0; tb < t1; tb += kChunk) {
     const int n = t1 - tb < kChunk ? t1 - tb : kChunk;
     __syncthreads();      // the chunk before is done with the operands, and S^T of its end is in LDS
     // q, k: SiLU, bfloat16; the weighted keys transposed.  v transposed.  Tokens beyond n are zeros.
-    for (int idx = threadIdx.x; idx < kChunk * DIM; idx += 256) {
-      const int j = idx / DIM, c = idx % DIM;
-      float qv = 0.f, kv = 0.f;
-      if (j < n) {
-        const float* row = proj + (size_t)(tb + j) * ld;
-        qv = silu_f(row[off_q + h * DIM + c]);
-        kv = silu_f(row[off_k + h * DIM + c]);
+#pragma unroll
+    for (int it = 0; it < NQ; ++it) {
+      const int idx = threadIdx.x + 256 * it, j = idx / RT, c = (idx % RT) * 4;
+      const float qa[4] = {rq[it].x, rq[it].y, rq[it].z, rq[it].w}, ka[4] = {rk[it].x, rk[it].y, rk[it].z, rk[it].w};
+      const float wj = j < n ? pow_int(l2, n - 1 - j) : 0.f;
+      uint16_t qb[4], kb[4];
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        qb[x] = bf16_of(j < n ? silu_fast(qa[x]) : 0.f);
+        kb[x] = bf16_of(j < n ? silu_fast(ka[x]) : 0.f);
+        const float kw = bf16_bits_to_f32(kb[x]) * wj;
+        const uint16_t hh = hi_of(kw);
+        Kth[(c + x) * TS + j] = hh;
+        Ktl[(c + x) * TS + j] = lo_of(kw, hh);
       }
-      const uint16_t kb = f32_to_bf16_bits(kv);
-      Qs[j * QS + c] = f32_to_bf16_bits(qv);
-      Ks[j * QS + c] = kb;
-      const float kw = j < n ? bf16_bits_to_f32(kb) * pow_int(l2, n - 1 - j) : 0.f;
-      const uint16_t hh = hi_of(kw);
-      Kth[c * TS + j] = hh;
-      Ktl[c * TS + j] = lo_of(kw, hh);
+      *reinterpret_cast<uint2*>(Qs + j * QS + c) = make_uint2(qb[0] | ((uint32_t)qb[1] << 16), qb[2] | ((uint32_t)qb[3] << 16));
+      *reinterpret_cast<uint2*>(Ks + j * QS + c) = make_uint2(kb[0] | ((uint32_t)kb[1] << 16), kb[2] | ((uint32_t)kb[3] << 16));
     }
-    for (int idx = threadIdx.x; idx < kChunk * kCols; idx += 256) {
-      const int j = idx / kCols, v = idx % kCols;
-      const float vv = (j < n && v0 + v < vdim) ? silu_f(proj[(size_t)(tb + j) * ld + off_v + h * vdim + v0 + v]) : 0.f;
-      Vt[v * TS + j] = f32_to_bf16_bits(vv);
+#pragma unroll
+    for (int it = 0; it < NV; ++it) {
+      const int idx = threadIdx.x + 256 * it, j = idx / kCols, v = idx % kCols;
+      Vt[v * TS + j] = bf16_of((j < n && v0 + v < vdim) ? silu_fast(rv[it]) : 0.f);
     }
+    if (tb + kChunk < t1) ask(tb + kChunk, t1 - tb - kChunk < kChunk ? t1 - tb - kChunk : kChunk);
     __syncthreads();
     // weighted scores of the wave's 16 tokens i against the keys j <= i: D[j][i] with A = K, B = Q
     const int i_in = w * 16 + r16;                       // the token this lane holds in every tile below

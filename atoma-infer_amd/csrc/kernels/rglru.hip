@@ -8,7 +8,7 @@
 // Everything behind the projection is float32.  A request's state row is [taps - 1][width] inputs of the convolution
 // (the latest last, biases included) followed by S [width]; zero at admission, which is "zeros before the start".
 //
-//   rglru_conv        a workgroup a token: u and g.  Inputs before the entry's first token come from the state row.
+//   rglru_conv        a thread a (token, channel): u and g.  Inputs before the entry's first token come from the state row.
 //   rglru_conv_state  a thread a (entry, channel): the state's inputs for the next step.
 //   rglru_scan        a thread a (entry, channel): the entry's tokens in order.
 //   long entries      S_t = a_t S_(t-1) + b_t is linear in S: rglru_stretch gives every (stretch of tokens, channel)
@@ -34,7 +34,8 @@ rglru_conv_kernel(const float* __restrict__ proj, int ld, int off_y, int off_x, 
   const int e = token_seq[t];
   const int i = t - q_start[e];                       // tokens of this entry before t
   const float* tail = state + (size_t)state_slots[e] * state_stride;
-  for (int c = threadIdx.x; c < width; c += 256) {
+  const int c = blockIdx.y * 256 + threadIdx.x;
+  if (c < width) {
     float acc = conv_b[c];
     for (int j = 0; j < taps; ++j) {
       const int back = taps - 1 - j;
@@ -168,7 +169,8 @@ extern "C" int atoma_rglru_conv(const float* proj, int ld, int off_y, int off_x,
       n_entries <= 0 || n_entries > 65535)
     return ATOMA_ERR_SHAPE;
   const size_t stride = (size_t)taps * width;      // taps - 1 rows of inputs, then S
-  hipLaunchKernelGGL(rglru_conv_kernel, dim3(n_tokens), dim3(256), 0, stream, proj, ld, off_y, off_x, by, bx, conv,
+  if ((width + 255) / 256 > 65535) return ATOMA_ERR_SHAPE;
+  hipLaunchKernelGGL(rglru_conv_kernel, dim3(n_tokens, (width + 255) / 256), dim3(256), 0, stream, proj, ld, off_y, off_x, by, bx, conv,
                      conv_b, token_seq, q_start, state_slots, state, stride, u, g, width, taps);
   if (taps > 1)
     hipLaunchKernelGGL(rglru_conv_state_kernel, dim3((width + 255) / 256, n_entries), dim3(256), 0, stream, proj, ld,

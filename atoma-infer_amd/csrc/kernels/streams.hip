@@ -29,7 +29,45 @@ struct StreamWeights {
   float in[kMaxStreams];
 };
 
-template <typename TY, typename TO, int SM>
+// V values of neighbouring columns at a time (V = 4: 16-byte loads of the copies, for rows of a multiple of 4 columns)
+template <int V> struct Vals {
+  float v[V];
+};
+template <int V> __device__ __forceinline__ Vals<V> load_vals(const float* p) {
+  Vals<V> r;
+  if constexpr (V == 4) {
+    const float4 q = *reinterpret_cast<const float4*>(p);
+    r.v[0] = q.x, r.v[1] = q.y, r.v[2] = q.z, r.v[3] = q.w;
+  } else {
+    r.v[0] = *p;
+  }
+  return r;
+}
+template <int V> __device__ __forceinline__ Vals<V> load_vals(const bf16_t* p) {
+  Vals<V> r;
+  if constexpr (V == 4) {
+    const uint2 q = *reinterpret_cast<const uint2*>(p);
+    r.v[0] = bf16_bits_to_f32(q.x & 0xffff), r.v[1] = bf16_bits_to_f32(q.x >> 16);
+    r.v[2] = bf16_bits_to_f32(q.y & 0xffff), r.v[3] = bf16_bits_to_f32(q.y >> 16);
+  } else {
+    r.v[0] = to_f32(*p);
+  }
+  return r;
+}
+template <int V> __device__ __forceinline__ void store_vals(float* p, const Vals<V>& a) {
+  if constexpr (V == 4) *reinterpret_cast<float4*>(p) = make_float4(a.v[0], a.v[1], a.v[2], a.v[3]);
+  else *p = a.v[0];
+}
+template <int V> __device__ __forceinline__ void store_vals(bf16_t* p, const Vals<V>& a) {
+  if constexpr (V == 4) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(f32_to_bf16_bits(a.v[0]) | ((uint32_t)f32_to_bf16_bits(a.v[1]) << 16),
+                                              f32_to_bf16_bits(a.v[2]) | ((uint32_t)f32_to_bf16_bits(a.v[3]) << 16));
+  } else {
+    *p = from_f32<bf16_t>(a.v[0]);
+  }
+}
+
+template <typename TY, typename TO, int SM, int V>
 __global__ void __launch_bounds__(256)
 stream_step_kernel(float* __restrict__ x, size_t copy_stride, int W, int S, const TY* __restrict__ y, int planes,
                    size_t plane_stride, const float* __restrict__ mix, const float* __restrict__ outw,
@@ -48,43 +86,65 @@ stream_step_kernel(float* __restrict__ x, size_t copy_stride, int W, int S, cons
   __syncthreads();
   float ss = 0.f;
   // (loops over the copies have the constant bound SM >= S, so that the copies' values stay in registers)
-  for (int c = threadIdx.x; c < W; c += 256) {
-    float old[SM], cur[SM];
+  for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+    Vals<V> old[SM], cur[SM];
 #pragma unroll
-    for (int s = 0; s < SM; ++s) old[s] = s < S ? x[s * copy_stride + (size_t)t * W + c] : 0.f;
+    for (int s = 0; s < SM; ++s) {
+      if (s < S) old[s] = load_vals<V>(x + s * copy_stride + (size_t)t * W + c);
+      else
+#pragma unroll
+        for (int e = 0; e < V; ++e) old[s].v[e] = 0.f;
+    }
     if (y) {
-      float yv = 0.f;
-      for (int p = 0; p < planes; ++p) yv += to_f32(y[p * plane_stride + (size_t)t * W + c]);
+      Vals<V> yv;
+#pragma unroll
+      for (int e = 0; e < V; ++e) yv.v[e] = 0.f;
+      for (int p = 0; p < planes; ++p) {
+        const Vals<V> a = load_vals<V>(y + p * plane_stride + (size_t)t * W + c);
+#pragma unroll
+        for (int e = 0; e < V; ++e) yv.v[e] += a.v[e];
+      }
 #pragma unroll
       for (int to = 0; to < SM; ++to) {
-        float v = 0.f;
 #pragma unroll
-        for (int s = 0; s < SM; ++s)
-          if (s < S && to < S) v = fmaf(sw.mix[s * S + to], old[s], v);
-        cur[to] = to < S ? fmaf(sw.out[to], yv, v) : 0.f;
+        for (int e = 0; e < V; ++e) {
+          float v = 0.f;
+#pragma unroll
+          for (int s = 0; s < SM; ++s)
+            if (s < S && to < S) v = fmaf(sw.mix[s * S + to], old[s].v[e], v);
+          cur[to].v[e] = to < S ? fmaf(sw.out[to], yv.v[e], v) : 0.f;
+        }
       }
       if (write_back) {
 #pragma unroll
         for (int s = 0; s < SM; ++s)
-          if (s < S) x[s * copy_stride + (size_t)t * W + c] = cur[s];
+          if (s < S) store_vals<V>(x + s * copy_stride + (size_t)t * W + c, cur[s]);
       }
     } else {
 #pragma unroll
       for (int s = 0; s < SM; ++s) cur[s] = old[s];
     }
     if (h) {
-      float u = 0.f;
 #pragma unroll
-      for (int s = 0; s < SM; ++s)
-        if (s < S) u = fmaf(sw.in[s], cur[s], u);
-      urow[c] = u;
-      ss = fmaf(u, u, ss);
+      for (int e = 0; e < V; ++e) {
+        float u = 0.f;
+#pragma unroll
+        for (int s = 0; s < SM; ++s)
+          if (s < S) u = fmaf(sw.in[s], cur[s].v[e], u);
+        urow[c + e] = u;
+        ss = fmaf(u, u, ss);
+      }
     }
   }
   if (!h) return;
   ss = block_sum<4>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)W + eps);
-  for (int c = threadIdx.x; c < W; c += 256) h[(size_t)r * W + c] = from_f32<TO>(urow[c] * inv * norm_w[c]);
+  for (int c = threadIdx.x * V; c < W; c += 256 * V) {
+    Vals<V> o;
+#pragma unroll
+    for (int e = 0; e < V; ++e) o.v[e] = urow[c + e] * inv * norm_w[c + e];
+    store_vals<V>(h + (size_t)r * W + c, o);
+  }
 }
 
 extern "C" int atoma_stream_step(float* x, int T, int W, int S, const void* y, int y_dtype, int planes,
@@ -97,13 +157,18 @@ extern "C" int atoma_stream_step(float* x, int T, int W, int S, const void* y, i
       (h && (!inw || !norm_w)))
     return ATOMA_ERR_SHAPE;
   const size_t copy_stride = (size_t)T * W, lds = h ? (size_t)W * 4 : 0;
-#define ATOMA_SS_N(TY, TO, SM)                                                                                    \
+#define ATOMA_SS_V(TY, TO, SM, V)                                                                                 \
   do {                                                                                                            \
     if (lds > 48 * 1024)                                                                                          \
-      (void)hipFuncSetAttribute((const void*)stream_step_kernel<TY, TO, SM>,                                      \
+      (void)hipFuncSetAttribute((const void*)stream_step_kernel<TY, TO, SM, V>,                                   \
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                            \
-    hipLaunchKernelGGL((stream_step_kernel<TY, TO, SM>), dim3(n), dim3(256), lds, stream, x, copy_stride, W, S,   \
+    hipLaunchKernelGGL((stream_step_kernel<TY, TO, SM, V>), dim3(n), dim3(256), lds, stream, x, copy_stride, W, S, \
                        (const TY*)y, planes, plane_stride, mix, outw, inw, norm_w, eps, (TO*)h, rows, write_back); \
+  } while (0)
+#define ATOMA_SS_N(TY, TO, SM)           \
+  do {                                   \
+    if (vec) ATOMA_SS_V(TY, TO, SM, 4);  \
+    else ATOMA_SS_V(TY, TO, SM, 1);      \
   } while (0)
 #define ATOMA_SS(TY, TO)                   \
   do {                                     \
@@ -112,6 +177,9 @@ extern "C" int atoma_stream_step(float* x, int T, int W, int S, const void* y, i
     else if (S <= 4) ATOMA_SS_N(TY, TO, 4); \
     else ATOMA_SS_N(TY, TO, 8);            \
   } while (0)
+  // rows of a multiple of 4 columns in tensors that torch allocated (aligned) take 16 bytes of a copy at a time
+  const bool vec = W % 4 == 0 && ((uintptr_t)x & 15) == 0 && ((uintptr_t)y & 15) == 0 && ((uintptr_t)h & 15) == 0 &&
+                   ((uintptr_t)norm_w & 15) == 0;
   const bool yb = y && y_dtype == kBF16, hb = h && h_dtype == kBF16;
   if (y && y_dtype != kF32 && y_dtype != kBF16) return ATOMA_ERR_DTYPE;
   if (h && h_dtype != kF32 && h_dtype != kBF16) return ATOMA_ERR_DTYPE;
@@ -121,6 +189,7 @@ extern "C" int atoma_stream_step(float* x, int T, int W, int S, const void* y, i
   else ATOMA_SS(float, float);
 #undef ATOMA_SS
 #undef ATOMA_SS_N
+#undef ATOMA_SS_V
   ATOMA_LAUNCH_CHECK();
   return 0;
 }
