@@ -58,7 +58,9 @@ tied_rope_prepare_kernel(const float* __restrict__ proj, int ld, int off_q, int 
   const int t = blockIdx.x;
   const float* p = proj + (size_t)t * ld;
   const int nq = nh * hd, nk = nkv * hd;
+#pragma unroll 8
   for (int i = threadIdx.x; i < nq; i += 256) row[i] = p[off_q + i] + (bq ? bq[i] : 0.f);
+#pragma unroll 4
   for (int i = threadIdx.x; i < nk; i += 256) row[nq + i] = p[off_k + i] + (bk ? bk[i] : 0.f);
   angles(positions[t], freq, rot, mag, cs, sn);
   __syncthreads();
@@ -68,6 +70,7 @@ tied_rope_prepare_kernel(const float* __restrict__ proj, int ld, int off_q, int 
     const float v = d >= hd ? 0.f : d < rot ? turned(x, d, rot, interleaved, cs, sn) : x[d];
     q_out[(size_t)t * nh * hd_out + i] = from_f32<TQ>(v);
   }
+#pragma unroll 8
   for (int i = threadIdx.x; i < nq; i += 256) gate[(size_t)t * nq + i] = 1.0f / (1.0f + expf(-p[off_g + i]));
   const int slot = slot_mapping[t];
   if (slot < 0) return;
@@ -103,6 +106,7 @@ latent_rope_prepare_kernel(const float* __restrict__ proj, int ld, int off_dq, i
   angles(positions[t], freq, rot, 1.0f, cs, sn);
   __syncthreads();
   for (int i = threadIdx.x; i < q_rank; i += 256) cq[(size_t)t * q_rank + i] = from_f32<TA>(p[off_dq + i] * iq * wq[i]);
+#pragma unroll 8
   for (int i = threadIdx.x; i < n_gate; i += 256) gate[(size_t)t * n_gate + i] = 1.0f / (1.0f + expf(-p[off_g + i]));
   const int slot = slot_mapping[t];
   if (slot < 0) return;
@@ -147,6 +151,7 @@ __global__ void __launch_bounds__(256)
 gate_mul_kernel(const TA* __restrict__ att, const float* __restrict__ gate, TA* __restrict__ y, int heads, int vd,
                 int hd_out) {
   const size_t t = blockIdx.x;
+#pragma unroll 8
   for (int i = threadIdx.x; i < heads * vd; i += 256) {
     const int h = i / vd, j = i % vd;
     y[t * heads * vd + i] = from_f32<TA>(to_f32(att[t * heads * hd_out + h * hd_out + j]) * gate[t * heads * vd + i]);

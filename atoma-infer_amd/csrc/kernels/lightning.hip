@@ -29,7 +29,7 @@ lightning_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off
                       const int32_t* __restrict__ q_start, const int32_t* __restrict__ state_slots,
                       float* __restrict__ state, const float* __restrict__ decay, float* __restrict__ o, int heads,
                       int dim, int vdim, int below) {
-  extern __shared__ float lds[];      // q [16][dim], k [16][dim], v [16][16]
+  extern __shared__ float lds[];      // q [16][dim], k [16][dim], v [16][16], the state's tile [16][dim]
   float* qs = lds;
   float* ks = lds + kLtTokens * dim;
   float* vs = ks + kLtTokens * dim;
@@ -42,12 +42,26 @@ lightning_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off
   const int j = vb * 16 + col;
   const bool live = j < vdim;
   const int rows = (dim + 15) / 16;
-  float* srow = state + ((size_t)state_slots[e] * heads + h) * (size_t)vdim * dim + (size_t)(live ? j : 0) * dim;
+  // The workgroup's columns of S are one stretch of memory (a column's rows are contiguous, and so are neighbouring
+  // columns): it is copied through LDS, 16 bytes a lane, so that the loads and stores of the state, which are most of
+  // what a decoded token moves, are whole cache lines; the lanes then pick their rows (part, part + 16, ...) from LDS.
+  float* stile = state + ((size_t)state_slots[e] * heads + h) * (size_t)vdim * dim + (size_t)vb * 16 * dim;
+  const int cols_live = vdim - vb * 16 < 16 ? vdim - vb * 16 : 16;
+  const int tile_n = cols_live * dim;
+  float* sbuf = vs + kLtTokens * 16;                     // [16][dim]
+  const bool vec = (dim & 3) == 0 && (((uintptr_t)stile) & 15) == 0;
+  if (vec) {
+    for (int i = threadIdx.x * 4; i < tile_n; i += 1024)
+      *reinterpret_cast<float4*>(sbuf + i) = *reinterpret_cast<const float4*>(stile + i);
+  } else {
+    for (int i = threadIdx.x; i < tile_n; i += 256) sbuf[i] = stile[i];
+  }
+  __syncthreads();
   float s[kLtMaxRows];
 #pragma unroll
   for (int i = 0; i < kLtMaxRows; ++i) {
     const int r = part + 16 * i;
-    s[i] = (live && i < rows && r < dim) ? srow[r] : 0.f;
+    s[i] = (live && i < rows && r < dim) ? sbuf[col * dim + r] : 0.f;
   }
   const float dec = decay[h];
   for (int tb = t0; tb < t1; tb += kLtTokens) {
@@ -83,12 +97,20 @@ lightning_scan_kernel(const float* __restrict__ proj, int ld, int off_q, int off
       if (part == 0 && live) o[(size_t)(tb + tt) * heads * vdim + h * vdim + j] = acc;
     }
   }
+  __syncthreads();
   if (live) {
 #pragma unroll
     for (int i = 0; i < kLtMaxRows; ++i) {
       const int r = part + 16 * i;
-      if (i < rows && r < dim) srow[r] = s[i];
+      if (i < rows && r < dim) sbuf[col * dim + r] = s[i];
     }
+  }
+  __syncthreads();
+  if (vec) {
+    for (int i = threadIdx.x * 4; i < tile_n; i += 1024)
+      *reinterpret_cast<float4*>(stile + i) = *reinterpret_cast<const float4*>(sbuf + i);
+  } else {
+    for (int i = threadIdx.x; i < tile_n; i += 256) stile[i] = sbuf[i];
   }
 }
 
@@ -323,9 +345,12 @@ lightning_out_kernel(const float* __restrict__ o, const float* __restrict__ proj
   __shared__ float scratch[4];
   const size_t t = blockIdx.x;
   float ss = 0.f;
+  // (unrolled: a thread's loads of a row are in flight together, which is what a step of few tokens waits for)
+#pragma unroll 8
   for (int c = threadIdx.x; c < n; c += 256) ss = fmaf(o[t * n + c], o[t * n + c], ss);
   ss = block_sum<4>(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+#pragma unroll 8
   for (int c = threadIdx.x; c < n; c += 256) {
     const float g = 1.0f / (1.0f + expf(-proj[t * ld + off_g + c]));
     y[t * n + c] = from_f32<TO>(o[t * n + c] * inv * w[c] * g);
@@ -338,19 +363,22 @@ static size_t chunk_lds(int dim) {
 }
 
 // chunked != 0: entries of at least `chunked` tokens run on the matrix cores (key sizes 32, 64, 96, 128 and decays
-// above zero only; the caller checks), the shorter ones token by token; 0: every entry token by token.
+// above zero only; the caller checks), the shorter ones token by token; 0: every entry token by token.  run_scan == 0:
+// the caller knows that no entry is shorter than `chunked` tokens, and the walk token by token is not launched.
 extern "C" int atoma_lightning_scan(const float* proj, int ld, int off_q, int off_k, int off_v, const int32_t* q_start,
                                     const int32_t* state_slots, float* state, const float* decay, float* o,
-                                    int n_entries, int heads, int dim, int vdim, int chunked, hipStream_t stream) {
+                                    int n_entries, int heads, int dim, int vdim, int chunked, int run_scan,
+                                    hipStream_t stream) {
   if (n_entries <= 0) return 0;
   if (heads <= 0 || dim <= 0 || dim > 16 * kLtMaxRows || vdim <= 0 || n_entries > 65535 || off_q < 0 || off_k < 0 ||
       off_v < 0 || ld < off_q + heads * dim || ld < off_k + heads * dim || ld < off_v + heads * vdim || chunked < 0 ||
       (chunked && (dim % 32 || dim > 128)))
     return ATOMA_ERR_SHAPE;
-  const size_t lds = (size_t)(2 * kLtTokens * dim + kLtTokens * 16) * sizeof(float);
+  const size_t lds = (size_t)(2 * kLtTokens * dim + kLtTokens * 16 + 16 * dim) * sizeof(float);
   dim3 grid(heads * ((vdim + 15) / 16), n_entries);
-  hipLaunchKernelGGL(lightning_scan_kernel, grid, dim3(256), lds, stream, proj, ld, off_q, off_k, off_v, q_start,
-                     state_slots, state, decay, o, heads, dim, vdim, chunked);
+  if (run_scan || !chunked)
+    hipLaunchKernelGGL(lightning_scan_kernel, grid, dim3(256), lds, stream, proj, ld, off_q, off_k, off_v, q_start,
+                       state_slots, state, decay, o, heads, dim, vdim, chunked);
   if (chunked) {
     const size_t clds = chunk_lds(dim) * sizeof(uint16_t);
     dim3 cgrid(heads * ((vdim + kCols - 1) / kCols), n_entries);

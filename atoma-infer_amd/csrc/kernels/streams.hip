@@ -205,25 +205,25 @@ bigram_embed_kernel(const int32_t* __restrict__ tokens, const int32_t* __restric
                     float scale, float* __restrict__ x, size_t copy_stride, int S, int W) {
   const int t = blockIdx.x;
   const int tok = tokens[t];
+  const int before = t > 0 ? tokens[t - 1] : 0;      // (asked for beside the rest; used inside an entry only)
   const int e = token_seq[t];
+  const int pos = positions[t];
   const int first = q_start[e], last = q_start[e + 1] - 1;
-  int prev = 0;
-  if (pairs) {
-    if (t == first) {
-      int32_t* st = state + state_slots[e];
-      prev = *st;
-      __syncthreads();      // every thread has read the row before one of them replaces it
-      if (threadIdx.x == 0) *st = tokens[last];
-    } else {
-      prev = tokens[t - 1];
-    }
+  int prev = before;
+  if (pairs && t == first) {
+    int32_t* st = state + state_slots[e];
+    const int32_t latest = tokens[last];
+    prev = *st;
+    __syncthreads();      // every thread has read the row before one of them replaces it
+    if (threadIdx.x == 0) *st = latest;
   }
   const bool ok = tok >= 0 && tok < vocab;
   long long row = buckets;
-  if (pairs && positions[t] > 0) {
+  if (pairs && pos > 0) {
     row = ((long long)prev * mul_prev + (long long)tok * mul_cur) % (long long)buckets;
     if (row < 0) row += buckets;
   }
+#pragma unroll 4
   for (int c = threadIdx.x; c < W; c += 256) {
     float v = __builtin_nanf("");
     if (ok) {
@@ -268,6 +268,7 @@ normed_branches_kernel(const TA* __restrict__ a, int planes_a, const TB* __restr
   __shared__ float scratch[4];
   const size_t t = blockIdx.x;
   float sa = 0.f, sb = 0.f;
+#pragma unroll 4
   for (int c = threadIdx.x; c < W; c += 256) {
     float va = bias_a ? bias_a[c] : 0.f, vb = bias_b ? bias_b[c] : 0.f;
     for (int p = 0; p < planes_a; ++p) va += to_f32(a[p * plane_stride + t * W + c]);
@@ -278,6 +279,7 @@ normed_branches_kernel(const TA* __restrict__ a, int planes_a, const TB* __restr
   sa = block_sum<4>(sa, scratch);
   sb = block_sum<4>(sb, scratch);
   const float ia = 1.0f / sqrtf(sa / (float)W + eps), ib = 1.0f / sqrtf(sb / (float)W + eps);
+#pragma unroll 4
   for (int c = threadIdx.x; c < W; c += 256)
     y[t * W + c] = scale * (rowbuf[c] * ia * wa[c] + rowbuf[W + c] * ib * wb[c]);
 }

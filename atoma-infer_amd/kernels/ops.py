@@ -1117,11 +1117,12 @@ def gate_mul(att: torch.Tensor, gate: torch.Tensor, heads: int, vd: int, hd_out:
 # -- recurrences with a decay per head or per channel -----------------------------------------------------------
 
 def lightning_scan(proj: torch.Tensor, offsets, q_start, state_slots, state: torch.Tensor, decay: torch.Tensor,
-                   heads: int, dim: int, vdim: int, chunked: int = 0) -> torch.Tensor:
+                   heads: int, dim: int, vdim: int, chunked: int = 0, scan: bool = True) -> torch.Tensor:
     """o float32 [T, heads vdim] of the recurrence S <- decay_h S + k v^T, o = S^T q over a step's entries; q, k, v are
     the SiLU of ``proj``'s columns at ``offsets`` = (q, k, v); each request's S is its row of ``state`` float32
     [slots, heads * vdim * dim].  ``chunked`` > 0: entries of at least that many tokens run 64 tokens at a time on the
-    matrix cores with q, k, v rounded to bfloat16 (key sizes 32, 64, 96, 128 and decays above zero only)."""
+    matrix cores with q, k, v rounded to bfloat16 (key sizes 32, 64, 96, 128 and decays above zero only); ``scan``
+    False then says that no entry is shorter, and the walk token by token is not launched."""
     _dev(proj, q_start, state_slots, state, decay)
     t = proj.shape[0]
     n_entries = state_slots.numel()
@@ -1140,8 +1141,8 @@ def lightning_scan(proj: torch.Tensor, offsets, q_start, state_slots, state: tor
     o = torch.empty((t, heads * vdim), dtype=torch.float32, device=proj.device)
     _check(_module("lightning").atoma_lightning_scan(_p(proj), proj.stride(0) if t > 1 else proj.shape[1], off_q, off_k,
                                                      off_v, _p(q_start), _p(state_slots), _p(state), _p(decay), _p(o),
-                                                     n_entries, heads, dim, vdim, int(chunked), _stream()),
-           "lightning_scan")
+                                                     n_entries, heads, dim, vdim, int(chunked), int(bool(scan)),
+                                                     _stream()), "lightning_scan")
     return o
 
 

@@ -356,8 +356,15 @@ class LightningAttention(Mixer):
         proj = linear(x, self.w_in, torch.float32)
         chunked = self.CHUNKED_FROM if (x.dtype is torch.bfloat16 and self.dim % 32 == 0 and self.dim <= 128
                                         and min(self.decay_list) > 0.0) else 0
+        # which of the two kernels a step needs follows from its entries' lengths, as its graph's key does
+        counts = getattr(ctx, "h_counts", None)
+        scan = True
+        if chunked and counts is not None and len(counts):
+            scan = int(counts.min()) < chunked
+            if int(counts.max()) < chunked:
+                chunked = 0
         o = ops.lightning_scan(proj, (0, self.off_k, self.off_v), ctx.q_start, ctx.state_slots, cache.state, self.decay,
-                               self.heads, self.dim, self.vdim, chunked)
+                               self.heads, self.dim, self.vdim, chunked, scan)
         y = ops.lightning_out(o, proj, self.off_g, self.norm_w, self.norm_eps, x.dtype)
         return linear_delta(y, self.w_o, None, self.w_o_tiled)
 
