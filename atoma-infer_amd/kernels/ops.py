@@ -852,9 +852,11 @@ def diff_combine(att: torch.Tensor, gate: torch.Tensor, heads: int, vdim: int, h
 MINGRU_STRETCH_MIN_TOKENS = 64      # entries of at least this many tokens are walked in stretches side by side
 
 
-def mingru_plan(counts, width: int, compute_units: int = 256):
+def mingru_plan(counts, width: int, compute_units: int = 256, min_length: int = 16):
     """The stretches of a step for ``mingru``: int32 [n][3] of (entry, first token, end) followed by [entries + 1] of
-    each entry's first stretch; None when no entry is long enough to pay for it.  A function of the entries' lengths."""
+    each entry's first stretch; None when no entry is long enough to pay for it.  A function of the entries' lengths.
+    ``min_length``: the shortest stretch (a recurrence whose walk over an entry's stretches costs two dependent loads
+    a stretch asks for longer ones)."""
     import numpy as np
     counts = np.asarray(counts, dtype=np.int64)
     if counts.size == 0 or int(counts.max()) < MINGRU_STRETCH_MIN_TOKENS:
@@ -863,7 +865,7 @@ def mingru_plan(counts, width: int, compute_units: int = 256):
     # times the channels' workgroups give every compute unit a few workgroups
     blocks = -(-width // 256)
     total = int(counts.sum())
-    length = max(16, min(256, (total * blocks) // (4 * compute_units)))
+    length = max(int(min_length), min(256, (total * blocks) // (4 * compute_units)))
     rows, first, t0 = [], [0], 0
     for e, c in enumerate(counts.tolist()):
         for lo in range(0, c, length):

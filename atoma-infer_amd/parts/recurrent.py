@@ -436,15 +436,17 @@ class GatedLinearRecurrence(Mixer):
     def device_bytes(self) -> int:
         return sum(w.numel() * w.element_size() for w in (self.w_in, self.w_gates, self.w_o))
 
+    MIN_STRETCH = 32
+
     def _plan_key(self):
-        return ("mingru_stretches", -(-self.inner // 256))
+        return ("rglru_stretches", -(-self.inner // 256))
 
     def step_planner(self, page_size: int, cache_dtype: torch.dtype):
         import numpy as np
         cus = torch.cuda.get_device_properties(self.w_o.device).multi_processor_count
 
         def plan(starts, counts, bucket):
-            got = ops.mingru_plan(counts, self.inner, cus)
+            got = ops.mingru_plan(counts, self.inner, cus, self.MIN_STRETCH)
             return got if got is not None else (np.zeros(0, dtype=np.int32), 0)
         return self._plan_key(), plan
 
@@ -455,7 +457,8 @@ class GatedLinearRecurrence(Mixer):
         gates = ops.head_linear(u, self.w_gates, torch.float32)
         plan = getattr(ctx, "plans", {}).get(self._plan_key())
         if plan is None and getattr(ctx, "h_counts", None) is not None:
-            got = ops.mingru_plan(ctx.h_counts, self.inner)      # a caller without a step planner: plan here and now
+            # a caller without a step planner: plan here and now
+            got = ops.mingru_plan(ctx.h_counts, self.inner, min_length=self.MIN_STRETCH)
             if got is not None:
                 plan = (torch.from_numpy(got[0]).to(x.device), got[1])
         y = ops.rglru_scan(gates, u, g, self.b_a, self.b_i, self.sp, ctx.q_start, ctx.state_slots, cache.state,
