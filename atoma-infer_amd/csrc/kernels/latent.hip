@@ -150,6 +150,35 @@ head_linear_mfma_kernel(const uint16_t* __restrict__ x, int ldx, const uint16_t*
   }
 }
 
+// The same for float32 rows of at most 16 tokens (the small products a decode step has): a wave an output column,
+// its lanes share the columns of K (coalesced reads of the weight's row), one sum per token, added over the lanes.
+template <typename TW>
+__global__ void __launch_bounds__(256)
+head_gemv_kernel(const float* __restrict__ x, int ldx, const TW* __restrict__ w, float* __restrict__ out, int ldo, int T,
+                 int H, int K, int N) {
+  const int lane = threadIdx.x & 63;
+  const long col = (long)blockIdx.x * 4 + (threadIdx.x >> 6);      // h * N + n
+  if (col >= (long)H * N) return;
+  const int h = (int)(col / N);
+  const TW* wr = w + (size_t)col * K;
+  float acc[16];
+#pragma unroll
+  for (int t = 0; t < 16; ++t) acc[t] = 0.f;
+  for (int k = lane; k < K; k += 64) {
+    const float wv = to_f32(wr[k]);
+#pragma unroll
+    for (int t = 0; t < 16; ++t)
+      if (t < T) acc[t] = fmaf(x[(size_t)t * ldx + (size_t)h * K + k], wv, acc[t]);
+  }
+#pragma unroll
+  for (int t = 0; t < 16; ++t) {
+    if (t < T) {
+      const float v = wave_sum(acc[t]);
+      if (lane == 0) out[(size_t)t * ldo + col] = v;
+    }
+  }
+}
+
 extern "C" int atoma_latent_prepare(const float* proj, int ldp, int off_q, int off_c, int off_g, int nq, int rank,
                                     int rank_p, int heads, const float* w_norm, float eps, void* kcache, void* vcache,
                                     int cache_dtype, const int32_t* slot_mapping, int page_size, void* q_out,
@@ -191,6 +220,19 @@ extern "C" int atoma_head_linear(const void* x, int x_dtype, int ldx, const void
       return ATOMA_ERR_DTYPE;
     }
 #undef ATOMA_HLM
+    ATOMA_LAUNCH_CHECK();
+    return 0;
+  }
+  if (T <= 16 && gate == nullptr && x_dtype == kF32 && out_dtype == kF32 && (long)H * N <= 4L * 2147483647L) {
+    const unsigned blocks = (unsigned)(((long)H * N + 3) / 4);
+    if (w_dtype == kF32)
+      hipLaunchKernelGGL((head_gemv_kernel<float>), dim3(blocks), dim3(256), 0, stream, (const float*)x, ldx,
+                         (const float*)w, (float*)out, ldo, T, H, K, N);
+    else if (w_dtype == kBF16)
+      hipLaunchKernelGGL((head_gemv_kernel<bf16_t>), dim3(blocks), dim3(256), 0, stream, (const float*)x, ldx,
+                         (const bf16_t*)w, (float*)out, ldo, T, H, K, N);
+    else
+      return ATOMA_ERR_DTYPE;
     ATOMA_LAUNCH_CHECK();
     return 0;
   }

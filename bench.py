@@ -333,10 +333,10 @@ def bafilorn_like(llama: dict, layers: int) -> dict:
            "mixer": {"left": {"dim": hd, "heads": nh, "kv_heads": nkv, "vdim": hd, "scale": hd ** -0.5,
                               "mask": {"size": 1024},
                               "rot": {"base": llama["rope_theta"], "dims": hd,
-                                      "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}}},
+                                      "scaling": {"factor": 8.0, "original": 8192, "fast": 16.0, "slow": 2.0}}},
                      "right": {"blocks": 16, "conv": 4, "width": w}}}
     kinds = [lat, lit, par, lit]
-    return {"architecture": "Bafilorn", "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 17}},
+    return {"architecture": "Bafilorn", "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 1000003, "mul_cur": 40503}},
             "layers": [kinds[i % 4] for i in range(layers)], "norm": {"eps": 1e-5}, "streams": 4,
             "loop": {"start": 0, "stop": layers, "times": 1}, "vocab": llama["vocab_size"], "width": w,
             "max_positions": llama["max_position_embeddings"]}
