@@ -2,6 +2,7 @@
 model's weights as numpy arrays."""
 from __future__ import annotations
 
+import math
 import os
 
 import numpy as np
@@ -82,6 +83,56 @@ BAF_D = config([
                                conv=2), 16),
     layer("lightning", lightning(heads=1, dim=1, vdim=1, decay=[0.9]), None),
 ], width=32, vocab=30, streams=1, bigram=(1, 5, 9), scale=2.0)
+
+
+def random_config(rng):
+    """A configuration drawn from ``rng`` (a ``random.Random``): two to eight layers of the three kinds in any order,
+    sizes that are and are not multiples of what the kernels like, every optional key present or absent."""
+    return rand_cfg(rng)
+
+
+def rand_cfg(rng):
+    width = rng.choice([96, 128, 192, 256, 320, 384])
+    kinds = ["latent_attention", "lightning", "parallel"]
+    n = rng.randint(2, 5)
+    order = [rng.choice(kinds) for _ in range(n)]
+    for k in kinds:
+        if k not in order and rng.random() < 0.7: order.append(k)
+    layers = []
+    for k in order:
+        ff = rng.choice([0, 64, 100, 256, 384]) if rng.random() < 0.85 else 0
+        if k == "latent_attention":
+            rd = rng.choice([0, 2, 8, 16, 32, 64])
+            rank = rng.choice([16, 24, 48, 96, 128, 160])
+            if rank + rd > 256: rank = 256 - rd
+            dims = rd if rng.random() < 0.7 else rng.choice([d for d in (0, 2, 4, 8, 16, 32) if d <= rd])
+            m = latent(dim=rng.choice([8, 16, 24, 32, 64]), heads=rng.choice([1, 2, 3, 4, 8, 12]), kv_rank=rank,
+                       q_rank=rng.choice([8, 32, 64, 128, 200]), rot_dim=rd, vdim=rng.choice([8, 16, 32, 48, 64]),
+                       scale=rng.choice([0.1, 0.15, 0.2]), base=rng.choice([100.0, 10000.0, 50000.0]), rot_dims=dims)
+        elif k == "lightning":
+            h = rng.choice([1, 2, 4, 6, 8])
+            m = lightning(heads=h, dim=rng.choice([8, 16, 32, 48, 64, 96, 128, 160]), vdim=rng.choice([8, 16, 24, 32, 64, 100]),
+                          decay=[math.exp(-1.0 / (2.0 ** (i + rng.random()))) if rng.random() < 0.9 else 0.999 for i in range(h)])
+        else:
+            kvh = rng.choice([1, 2, 4])
+            g = rng.choice([1, 2, 4, 8])
+            dim = rng.choice([16, 32, 40, 64, 80, 128])
+            rot = rng.choice([0, 8, 16, dim])
+            if rot > dim: rot = dim
+            sc = None if rng.random() < 0.3 else (rng.choice([2.0, 4.0, 8.0, 16.0]), rng.choice([64, 512, 2048, 4096]), rng.choice([8.0, 32.0, 64.0]), rng.choice([0.5, 1.0, 2.0]))
+            bw = rng.choice([64, 128, 256, 96])
+            blocks = rng.choice([b for b in (1, 2, 4, 8, 3) if bw % b == 0])
+            m = parallel(dim=dim, heads=kvh * g, kv_heads=kvh, scale=rng.choice([0.125, 0.1, 0.2]), mask=rng.choice([None, 5, 16, 37, 64, 100, 150]),
+                         rot_dims=rot, base=rng.choice([1000.0, 30000.0, 500000.0]), scaling=sc if rot else None, width=bw, blocks=blocks,
+                         conv=rng.choice([1, 2, 3, 4, 5, 7]))
+        layers.append(layer(k, m, ff))
+    loop = None
+    if rng.random() < 0.7:
+        a = rng.randint(0, len(layers) - 1); b = rng.randint(a + 1, len(layers))
+        loop = (a, b, rng.choice([1, 2, 3]))
+    bg = None if rng.random() < 0.2 else (rng.choice([7, 101, 521, 4099]), rng.choice([1, 29, 1009, 65537]), rng.choice([1, 19, 257, 40503]))
+    return config(layers, width=width, vocab=rng.choice([50, 97, 300, 450, 1000]), eps=rng.choice([1e-6, 1e-5]),
+                  streams=rng.choice([None, 1, 2, 3, 4, 5]), bigram=bg, scale=rng.choice([1.0, 10.0, 0.5]), loop=loop)
 
 
 def numpy_weights(path: str):

@@ -115,9 +115,12 @@ def latent_attention(h, p, w, pre, m, eps):
     dkv = h @ w[pre + "dkv"].T
     c = unit_rms(dkv[:, :kr], eps) * w[pre + "dkv.norm"]
     k_rot = dkv[:, kr:].reshape(T, 1, r)
-    f = plain_frequencies(m["rot"]["base"], m["rot"]["dims"])
-    q_rot = rotate(q[..., d:], p, f, m["rot"]["dims"], "interleaved")
-    k_rot = rotate(k_rot, p, f, m["rot"]["dims"], "interleaved")
+    q_rot = q[..., d:]
+    rot = m.get("rot")
+    if rot is not None and rot["dims"]:
+        f = plain_frequencies(rot["base"], rot["dims"])
+        q_rot = rotate(q_rot, p, f, rot["dims"], "interleaved")
+        k_rot = rotate(k_rot, p, f, rot["dims"], "interleaved")
     k = np.concatenate([(c @ w[pre + "uk"].T).reshape(T, H, d), np.repeat(k_rot, H, axis=1)], axis=2)
     v = (c @ w[pre + "uv"].T).reshape(T, H, dv)
     qq = np.concatenate([q[..., :d], q_rot], axis=2)
@@ -135,7 +138,7 @@ def tied_value_attention(h, p, w, pre, m):
     k = (h @ w[pre + "k"].T + w[pre + "k.b"]).reshape(T, G, d)
     v = k.copy()
     rot = m.get("rot")
-    if rot is not None:
+    if rot is not None and rot["dims"]:
         f, mag = yarn_frequencies(rot["base"], rot["dims"], rot.get("scaling"))
         q = rotate(q, p, f, rot["dims"], "half", mag)
         k = rotate(k, p, f, rot["dims"], "half", mag)
